@@ -1,0 +1,100 @@
+/* C ABI of libpbs_hip.so -- the gfx950 (MI355X) kernels behind PBS-Attn's
+ * permuted block-sparse prefill attention.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless named otherwise; tensors are bf16
+ *     (uint16 storage) with head_dim 128 and block_size 128;
+ *   - strides are in ELEMENTS (batch, head, sequence); the innermost dimension has
+ *     stride 1 and every row must start 16-byte aligned;
+ *   - K/V may be given at Hkv heads (query head h reads KV head h / (Hq / Hkv)) or
+ *     already repeated to Hq heads (pass Hkv = Hq);
+ *   - `stream` is a hipStream_t; all work is enqueued on it, nothing synchronises,
+ *     nothing allocates; scratch memory comes in through `workspace`;
+ *   - return 0 on success, a negative value for an argument error, a positive
+ *     hipError_t for a launch error; pbs_last_error() gives the message (thread local).
+ *
+ * File:line citations name the reference code (xinghaow99/pbs-attn) each entry
+ * point replaces.
+ */
+#ifndef PBS_HIP_H
+#define PBS_HIP_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+int pbs_abi_version(void);
+const char* pbs_last_error(void);
+
+/* Key scoring: scores[b,h,k] = mean over the last 128 queries of
+ * softmax_k(bf16(bf16(q.k) / sqrt(D))) over the keys of the complete segments.
+ * scores: (B, Hq, Sc) float32, Sc = (S / segment_size) * segment_size.
+ * Replaces pbs_attn/src/permute_states.py:44-50. */
+size_t pbs_score_keys_workspace_bytes(int B, int Hq, int S, int segment_size);
+int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
+                   int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
+                   int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Per-segment stable descending argsort (ties keep ascending index).
+ * scores: (rows, Sc); key_indices: (rows, S_pad) int32 global key positions;
+ * positions >= Sc (trailing partial segment, block padding) keep identity order.
+ * Replaces pbs_attn/src/permute_states.py:52-56,71-81 and the index padding of
+ * pbs_attn/src/pbs.py:80-84. */
+int pbs_segment_argsort(const float* scores, int32_t* key_indices, int rows, int S, int S_pad, int segment_size,
+                        void* stream);
+
+/* Gather K and V into permuted order and pool the permuted key blocks.
+ * perm_k: (B, Hq, nb*128, 128) rows past S zero; perm_vt: (B, Hq, nb, 128, 128)
+ * holding each V block transposed [d][key]; pooled_k: (B, Hq, nb, 128) bf16.
+ * Replaces pbs_attn/src/permute_states.py:59-69, pbs_attn/src/pbs.py:213-215,
+ * the key padding of pbs.py:78-79 and the key pooling of pbs_attn/src/utils.py:24-29. */
+int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
+                  void* pooled_k, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
+                  int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
+                  void* stream);
+
+/* Query-block pooling (mean with divisor 128, or max; rows past S count as zero).
+ * pooled_q: (B, Hq, nb, 128) bf16.  Replaces pbs_attn/src/pbs.py:67-71 and
+ * pbs_attn/src/utils.py:18-23. */
+int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim, int block_size, int64_t q_sb,
+               int64_t q_sh, int64_t q_ss, int query_pool_max, void* stream);
+
+/* Block logits + masked fp32 softmax.  block_attn_scores: (rows, nb, nb) float32;
+ * candidates of query block qb are the key blocks of strictly earlier segments;
+ * rows without candidates are NaN.  Replaces pbs_attn/src/pbs.py:97-107 and
+ * pbs_attn/src/utils.py:30-33. */
+int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows, int nb,
+                             int head_dim, int blocks_per_segment, void* stream);
+
+/* Cumulative-threshold selection.  threshold_per_row (rows floats) overrides
+ * `threshold` when non-null; threshold_is_int_one selects every candidate.
+ * sel_mask = selected | first-token block; final_mask = sel_mask | own segment
+ * (both (rows, nb, nb) bytes, either may be null); csr_cols (rows, nb, nb) /
+ * csr_cnt (rows, nb): ascending key blocks the attention kernel visits.
+ * Replaces pbs_attn/src/utils.py:38-86 and pbs_attn/src/pbs.py:10-25,119-127,209. */
+size_t pbs_select_blocks_workspace_bytes(int rows);
+int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
+                      int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices, int rows,
+                      int S, int block_size, int segment_size, uint8_t* sel_mask, uint8_t* final_mask,
+                      int32_t* csr_cols, int32_t* csr_cnt, void* workspace, size_t workspace_bytes, void* stream);
+
+/* Block-sparse flash-attention forward over the permuted K / transposed V tiles.
+ * out: (B, Hq, S, 128) bf16 with its own strides, original query order.
+ * Replaces pbs_attn/src/kernels/permuted_block_sparse_attention.py:134-311
+ * (launch at pbs_attn/src/pbs.py:220-246). */
+int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const int32_t* key_indices,
+                        const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int S,
+                        int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                        int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale, void* stream);
+
+/* out[b,h,q_idx[b,h,i],:] = o_perm[b,h,i,:] (o_perm contiguous).  q_idx null with
+ * o_perm == out is the identity fast path (no launch): the reference does not
+ * permute queries (pbs_attn/src/pbs.py:191-193), so this is what it takes. */
+int pbs_unpermute(const void* o_perm, const int32_t* q_idx, void* out, int B, int H, int S, int head_dim,
+                  int64_t o_sb, int64_t o_sh, int64_t o_ss, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,54 @@
+"""Builds libpbs_hip.so (the gfx950 kernels + C ABI) in-tree with hipcc."""
+from __future__ import annotations
+
+import os
+import shutil
+import subprocess
+import tempfile
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(HERE, "csrc")
+LIB_DIR = os.path.join(HERE, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libpbs_hip.so")
+
+SOURCES = ["pbs_abi.hip", "pbs_score.hip", "pbs_sort.hip", "pbs_gather.hip", "pbs_estimate.hip",
+           "pbs_select.hip", "pbs_attn.hip"]
+
+DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
+                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+                "-Wno-unused-command-line-argument", "-Wno-unused-value"]
+
+
+def _hipcc() -> str:
+    exe = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(exe):
+        raise RuntimeError("hipcc not found: the PBS HIP kernels cannot be built")
+    return exe
+
+
+def build_library(verbose: bool = False) -> str:
+    """Compiles every .hip source for gfx950 and links the shared library."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = _hipcc()
+    with tempfile.TemporaryDirectory() as tmp:
+        objs = []
+        procs = []
+        for src in SOURCES:
+            obj = os.path.join(tmp, src.replace(".hip", ".o"))
+            cmd = [hipcc, *DEVICE_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+            procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
+            objs.append(obj)
+        for src, p in procs:
+            out, err = p.communicate()
+            if p.returncode != 0:
+                raise RuntimeError(f"hipcc failed on {src}:\n{err}")
+            if verbose and err.strip():
+                print(err)
+        tmp_lib = os.path.join(tmp, "libpbs_hip.so")
+        subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp_lib, *objs], check=True)
+        shutil.move(tmp_lib, LIB_PATH)
+    return LIB_PATH
+
+
+if __name__ == "__main__":
+    print(build_library(verbose=True))

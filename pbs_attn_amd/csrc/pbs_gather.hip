@@ -1,0 +1,169 @@
+// Gather of K and V into permuted order, fused with the key-block pooling.
+//
+// One workgroup moves one block of 128 permuted keys of one head:
+//   perm_k  (B, Hq, nb*128, 128)   row-major, rows past S are zero
+//   perm_vt (B, Hq, nb, 128, 128)  V block TRANSPOSED: [d][key in block] -- the
+//                                  layout the attention kernel feeds to MFMA
+//   pooled_k(B, Hq, nb, 128)       bf16 mean (fp32 accumulate / 128) or max
+// A 256-byte source row is read by 16 lanes x 16 bytes; K/V may be stored at
+// the KV-head count (query head h reads KV head h / G).
+#include "pbs_common.h"
+
+namespace {
+
+constexpr int D = 128;
+constexpr int BS = 128;
+constexpr int VT_PITCH = 130;  // bf16 elements per staged V row (padded: bank spread)
+
+struct GatherArgs {
+  const uint16_t* k;
+  const uint16_t* v;
+  const int32_t* idx;  // (B*Hq, S_pad)
+  uint16_t* perm_k;
+  uint16_t* perm_vt;
+  uint16_t* pooled_k;
+  int B, Hq, Hkv, S, nb;
+  int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
+  int pool_max;
+};
+
+__global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
+  __shared__ uint16_t vt[BS * VT_PITCH];
+  __shared__ float pool[16][D];
+  const int kb = blockIdx.x, bh = blockIdx.y;
+  const int b = bh / a.Hq, h = bh % a.Hq, kvh = h / (a.Hq / a.Hkv);
+  const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;  // row group, 16-byte chunk
+  const uint16_t* ksrc = a.k + b * a.k_sb + kvh * a.k_sh;
+  const uint16_t* vsrc = a.v + b * a.v_sb + kvh * a.v_sh;
+  const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS + kb * BS;
+  uint16_t* kdst = a.perm_k + ((int64_t)bh * a.nb + kb) * BS * D;
+
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = a.pool_max ? -INFINITY : 0.f;
+
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int i = pass * 16 + rg;
+    const int pos = kb * BS + i;
+    u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+    if (pos < a.S) {
+      const int src = idx[i];
+      kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
+      vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
+    }
+    *reinterpret_cast<u32x4*>(kdst + i * D + c * 8) = kv;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = bf16_bits_to_f32(kv[e] & 0xffffu), hi = bf16_bits_to_f32(kv[e] >> 16);
+      if (a.pool_max) {
+        acc[2 * e] = fmaxf(acc[2 * e], lo);
+        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], hi);
+      } else {
+        acc[2 * e] += lo;
+        acc[2 * e + 1] += hi;
+      }
+      // stage V row-major (4-byte stores: the padded pitch keeps them aligned)
+      *reinterpret_cast<uint32_t*>(&vt[i * VT_PITCH + c * 8 + 2 * e]) = vv[e];
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) pool[rg][c * 8 + e] = acc[e];
+  __syncthreads();
+
+  if (threadIdx.x < D) {
+    float s = pool[0][threadIdx.x];
+    for (int r = 1; r < 16; ++r) s = a.pool_max ? fmaxf(s, pool[r][threadIdx.x]) : s + pool[r][threadIdx.x];
+    if (!a.pool_max) s = s / (float)BS;
+    a.pooled_k[((int64_t)bh * a.nb + kb) * D + threadIdx.x] = (uint16_t)f32_to_bf16_bits(s);
+  }
+
+  // transposed write-out: thread (d, key group of 8) -> 16 bytes of row d
+  uint16_t* vdst = a.perm_vt + ((int64_t)bh * a.nb + kb) * D * BS;
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int d = pass * 16 + rg;
+    u32x4 o;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t lo = vt[(c * 8 + 2 * e) * VT_PITCH + d], hi = vt[(c * 8 + 2 * e + 1) * VT_PITCH + d];
+      o[e] = lo | (hi << 16);
+    }
+    *reinterpret_cast<u32x4*>(vdst + d * BS + c * 8) = o;
+  }
+}
+
+// Mean / max pooling of Q blocks (rows past S count as zeros, the divisor stays 128).
+__global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t* pooled, int Hq, int S, int nb,
+                                                     int64_t q_sb, int64_t q_sh, int64_t q_ss, int pool_max) {
+  __shared__ float pool[16][D];
+  const int qb = blockIdx.x, bh = blockIdx.y;
+  const int b = bh / Hq, h = bh % Hq;
+  const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;
+  const uint16_t* src = q + b * q_sb + h * q_sh;
+  float acc[8];
+#pragma unroll
+  for (int e = 0; e < 8; ++e) acc[e] = pool_max ? -INFINITY : 0.f;
+#pragma unroll
+  for (int pass = 0; pass < 8; ++pass) {
+    const int pos = qb * BS + pass * 16 + rg;
+    u32x4 x = {0, 0, 0, 0};
+    if (pos < S) x = *reinterpret_cast<const u32x4*>(src + (int64_t)pos * q_ss + c * 8);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float lo = bf16_bits_to_f32(x[e] & 0xffffu), hi = bf16_bits_to_f32(x[e] >> 16);
+      if (pool_max) {
+        acc[2 * e] = fmaxf(acc[2 * e], lo);
+        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], hi);
+      } else {
+        acc[2 * e] += lo;
+        acc[2 * e + 1] += hi;
+      }
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 8; ++e) pool[rg][c * 8 + e] = acc[e];
+  __syncthreads();
+  if (threadIdx.x < D) {
+    float s = pool[0][threadIdx.x];
+    for (int r = 1; r < 16; ++r) s = pool_max ? fmaxf(s, pool[r][threadIdx.x]) : s + pool[r][threadIdx.x];
+    if (!pool_max) s = s / (float)BS;
+    pooled[((int64_t)bh * nb + qb) * D + threadIdx.x] = (uint16_t)f32_to_bf16_bits(s);
+  }
+}
+
+}  // namespace
+
+extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
+                             void* pooled_k, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
+                             int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
+                             void* stream) {
+  PBS_REQUIRE(k && v && key_indices && perm_k && perm_vt && pooled_k, "pbs_gather_kv: null tensor pointer");
+  PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_gather_kv: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
+  PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_gather_kv: bad shape");
+  PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_ss % 8 == 0,
+              "pbs_gather_kv: strides must keep rows 16-byte aligned");
+  PBS_REQUIRE(((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0, "pbs_gather_kv: pointers must be 16-byte aligned");
+  PBS_REQUIRE(B * Hq <= 65535, "pbs_gather_kv: too many heads");
+  GatherArgs a;
+  a.k = (const uint16_t*)k; a.v = (const uint16_t*)v; a.idx = key_indices;
+  a.perm_k = (uint16_t*)perm_k; a.perm_vt = (uint16_t*)perm_vt; a.pooled_k = (uint16_t*)pooled_k;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
+  a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss; a.v_sb = v_sb; a.v_sh = v_sh; a.v_ss = v_ss;
+  a.pool_max = key_pool_max;
+  hipLaunchKernelGGL(gather_kv_kernel, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
+  return pbs_check_launch("pbs_gather_kv");
+}
+
+extern "C" int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim, int block_size,
+                          int64_t q_sb, int64_t q_sh, int64_t q_ss, int query_pool_max, void* stream) {
+  PBS_REQUIRE(q && pooled_q, "pbs_pool_q: null tensor pointer");
+  PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_pool_q: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
+  PBS_REQUIRE(B > 0 && Hq > 0 && S > 0 && B * Hq <= 65535, "pbs_pool_q: bad shape");
+  PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && ((uintptr_t)q % 16) == 0,
+              "pbs_pool_q: rows must be 16-byte aligned");
+  const int nb = (S + BS - 1) / BS;
+  hipLaunchKernelGGL(pool_q_kernel, dim3(nb, B * Hq), dim3(256), 0, (hipStream_t)stream, (const uint16_t*)q,
+                     (uint16_t*)pooled_q, Hq, S, nb, q_sb, q_sh, q_ss, query_pool_max);
+  return pbs_check_launch("pbs_pool_q");
+}

@@ -1,0 +1,211 @@
+// Key scoring: mean over the last 128 queries of softmax(Q_last K^T / sqrt(D))
+// over all keys of the complete segments (no causal mask).
+//
+// Three launches, K is read twice and never re-materialised:
+//   1. score_partial : per (head, key chunk) online (max, sum-exp) of every query row
+//   2. score_reduce  : fold the chunk partials into (row max, 1 / row sum)
+//   3. score_final   : recompute the logits and emit the per-key mean probability
+// Logits reproduce the rounding points of a bf16 matmul followed by a bf16
+// divide: fp32 accumulate -> bf16 -> / sqrt(D) -> bf16.
+#include "pbs_common.h"
+
+namespace {
+
+constexpr int D = 128;             // head dim
+constexpr int NQ = 128;            // scoring queries (= block size)
+constexpr int KEYS_PER_WAVE_STEP = 32;
+constexpr int KEYS_PER_WG = 1024;  // keys one 4-wave workgroup walks through (256 for 1-wave groups)
+
+struct ScoreArgs {
+  const uint16_t* q;
+  const uint16_t* k;
+  int B, Hq, Hkv, S, Sc;
+  int64_t q_sb, q_sh, q_ss;
+  int64_t k_sb, k_sh, k_ss;
+  float sqrt_d;
+  float* part;    // (B*Hq, nchunk, NQ, 2)
+  float* stats;   // (B*Hq, NQ, 2)  (max, 1/sum)
+  float* scores;  // (B*Hq, Sc)
+  int nchunk;
+  int chunk_keys;
+};
+
+__device__ __forceinline__ bf16x8 load_frag(const uint16_t* row_ptr, int t, int half) {
+  return *reinterpret_cast<const bf16x8*>(row_ptr + 16 * t + 8 * half);
+}
+
+__device__ __forceinline__ float logit_round(float acc, float sqrt_d) {
+  return round_bf16(round_bf16(acc) / sqrt_d);
+}
+
+// One wave per query head of the KV group; the four waves of a workgroup walk
+// the same key chunk so K comes out of the CU's L1 after the first wave.
+template <bool FINAL>
+__global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int j = lane & 31, half = lane >> 5;
+  const int G = a.Hq / a.Hkv;
+  const int b = blockIdx.y / a.Hkv, kvh = blockIdx.y % a.Hkv;
+  const int chunk = blockIdx.x;
+  const int key_lo = chunk * a.chunk_keys;
+  const int key_hi = min(key_lo + a.chunk_keys, a.Sc);
+  const int nwaves = blockDim.x >> 6;
+  const uint16_t* kbase = a.k + b * a.k_sb + kvh * a.k_sh;
+
+  __shared__ float s_stats[4][NQ][2];
+
+  for (int g0 = 0; g0 < G; g0 += nwaves) {
+    const int g = g0 + wave;
+    const bool active = g < G;
+    const int h = kvh * G + (active ? g : 0);
+    const int bh = b * a.Hq + h;
+    const uint16_t* qbase = a.q + b * a.q_sb + h * a.q_sh + (int64_t)(a.S - NQ) * a.q_ss;
+
+    // the head's 128 scoring queries, resident for the whole chunk
+    bf16x8 qf[4][8];
+#pragma unroll
+    for (int qt = 0; qt < 4; ++qt)
+#pragma unroll
+      for (int t = 0; t < 8; ++t) qf[qt][t] = load_frag(qbase + (int64_t)(32 * qt + j) * a.q_ss, t, half);
+
+    if (FINAL) {
+      __syncthreads();
+      if (active)
+        for (int i = lane; i < NQ * 2; i += 64) (&s_stats[wave][0][0])[i] = a.stats[(int64_t)bh * NQ * 2 + i];
+      __syncthreads();
+    }
+
+    float m_run[4], l_run[4];
+#pragma unroll
+    for (int qt = 0; qt < 4; ++qt) {
+      m_run[qt] = -INFINITY;
+      l_run[qt] = 0.f;
+    }
+
+    if (active) {
+      for (int key0 = key_lo; key0 < key_hi; key0 += KEYS_PER_WAVE_STEP) {
+        const int key = key0 + j;  // always < Sc: Sc is a multiple of 128
+        const uint16_t* krow = kbase + (int64_t)key * a.k_ss;
+        bf16x8 kf[8];
+#pragma unroll
+        for (int t = 0; t < 8; ++t) kf[t] = load_frag(krow, t, half);
+
+        if (!FINAL) {
+          // S^T tile: rows = keys, column = query j of sub-tile qt
+#pragma unroll
+          for (int qt = 0; qt < 4; ++qt) {
+            f32x16 acc = {0};
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t], qf[qt][t], acc, 0, 0, 0);
+            float v[16], mx = -INFINITY;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              v[r] = logit_round(acc[r], a.sqrt_d);
+              mx = fmaxf(mx, v[r]);
+            }
+            const float m_new = fmaxf(m_run[qt], mx);
+            float sum = 0.f;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sum += __expf(v[r] - m_new);
+            l_run[qt] = l_run[qt] * __expf(m_run[qt] - m_new) + sum;
+            m_run[qt] = m_new;
+          }
+        } else {
+          // S tile: rows = queries of sub-tile qt, column = key j
+          float accp = 0.f;
+#pragma unroll
+          for (int qt = 0; qt < 4; ++qt) {
+            f32x16 acc = {0};
+#pragma unroll
+            for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[qt][t], kf[t], acc, 0, 0, 0);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              const int qrow = 32 * qt + 8 * (r >> 2) + 4 * half + (r & 3);
+              const float mx = s_stats[wave][qrow][0], inv = s_stats[wave][qrow][1];
+              accp += __expf(logit_round(acc[r], a.sqrt_d) - mx) * inv;
+            }
+          }
+          accp += xhalf_f32(accp);
+          if (half == 0) a.scores[(int64_t)bh * a.Sc + key] = accp * (1.0f / NQ);
+        }
+      }
+      if (!FINAL) {
+#pragma unroll
+        for (int qt = 0; qt < 4; ++qt) {
+          const float m_o = xhalf_f32(m_run[qt]), l_o = xhalf_f32(l_run[qt]);
+          const float m_new = fmaxf(m_run[qt], m_o);
+          const float l_new = l_run[qt] * __expf(m_run[qt] - m_new) + l_o * __expf(m_o - m_new);
+          if (half == 0) {
+            float* p = a.part + (((int64_t)bh * a.nchunk + chunk) * NQ + 32 * qt + j) * 2;
+            p[0] = m_new;
+            p[1] = l_new;
+          }
+        }
+      }
+    }
+  }
+}
+
+__global__ __launch_bounds__(NQ) void score_reduce_kernel(ScoreArgs a) {
+  const int bh = blockIdx.x, qrow = threadIdx.x;
+  const float* p = a.part + (int64_t)bh * a.nchunk * NQ * 2;
+  float m = -INFINITY, l = 0.f;
+  for (int c = 0; c < a.nchunk; ++c) {
+    const float mc = p[((int64_t)c * NQ + qrow) * 2], lc = p[((int64_t)c * NQ + qrow) * 2 + 1];
+    const float m_new = fmaxf(m, mc);
+    l = l * __expf(m - m_new) + lc * __expf(mc - m_new);
+    m = m_new;
+  }
+  a.stats[((int64_t)bh * NQ + qrow) * 2] = m;
+  a.stats[((int64_t)bh * NQ + qrow) * 2 + 1] = 1.0f / l;
+}
+
+// With one query head per KV head a workgroup is a single wave and takes a
+// quarter of the keys, so the launch still fills the chip.
+int chunk_keys_for(int G) { return G > 1 ? KEYS_PER_WG : KEYS_PER_WG / 4; }
+int chunks_for(int Sc, int chunk_keys) { return (Sc + chunk_keys - 1) / chunk_keys; }
+
+}  // namespace
+
+extern "C" size_t pbs_score_keys_workspace_bytes(int B, int Hq, int S, int segment_size) {
+  if (segment_size <= 0) return 0;
+  const int Sc = (S / segment_size) * segment_size;
+  return (size_t)B * Hq * ((size_t)chunks_for(Sc, KEYS_PER_WG / 4) + 1) * NQ * 2 * sizeof(float);
+}
+
+extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
+                              int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
+                              int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream) {
+  PBS_REQUIRE(q && k && scores, "pbs_score_keys: null tensor pointer");
+  PBS_REQUIRE(head_dim == D, "pbs_score_keys: head_dim must be 128, got %d", head_dim);
+  PBS_REQUIRE(block_size == NQ, "pbs_score_keys: block_size must be 128, got %d", block_size);
+  PBS_REQUIRE(B > 0 && Hkv > 0 && Hq > 0 && Hq % Hkv == 0, "pbs_score_keys: bad head counts Hq=%d Hkv=%d", Hq, Hkv);
+  PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_score_keys: segment_size %d not a multiple of block_size", segment_size);
+  PBS_REQUIRE(S >= NQ, "pbs_score_keys: sequence shorter than one block");
+  PBS_REQUIRE(q_ss % 8 == 0 && k_ss % 8 == 0 && q_sh % 8 == 0 && k_sh % 8 == 0 && q_sb % 8 == 0 && k_sb % 8 == 0,
+              "pbs_score_keys: strides must keep rows 16-byte aligned");
+  PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0, "pbs_score_keys: pointers must be 16-byte aligned");
+  const int Sc = (S / segment_size) * segment_size;
+  if (Sc == 0) return 0;
+  PBS_REQUIRE(workspace && workspace_bytes >= pbs_score_keys_workspace_bytes(B, Hq, S, segment_size),
+              "pbs_score_keys: workspace too small");
+  ScoreArgs a;
+  a.q = (const uint16_t*)q;
+  a.k = (const uint16_t*)k;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.Sc = Sc;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss;
+  a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
+  a.sqrt_d = (float)sqrt((double)head_dim);
+  a.chunk_keys = chunk_keys_for(Hq / Hkv);
+  a.nchunk = chunks_for(Sc, a.chunk_keys);
+  a.part = (float*)workspace;
+  a.stats = a.part + (size_t)B * Hq * a.nchunk * NQ * 2;
+  a.scores = scores;
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid(a.nchunk, B * Hkv);
+  const dim3 block(Hq / Hkv > 1 ? 256 : 64);
+  hipLaunchKernelGGL(score_kernel<false>, grid, block, 0, st, a);
+  hipLaunchKernelGGL(score_reduce_kernel, dim3(B * Hq), dim3(NQ), 0, st, a);
+  hipLaunchKernelGGL(score_kernel<true>, grid, block, 0, st, a);
+  return pbs_check_launch("pbs_score_keys");
+}

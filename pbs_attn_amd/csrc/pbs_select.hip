@@ -1,0 +1,171 @@
+// Cumulative-threshold block selection and CSR emission.
+//
+// One workgroup per (head, query block) row of the block-probability matrix:
+//   * NaN -> 0, stable descending sort of the row in LDS (64-bit composite keys),
+//   * running sum in the order torch's CPU cumsum uses: sequential, accumulated in
+//     float64, every prefix rounded to float32 and compared with float32(threshold),
+//   * keep ranks <= the first prefix that reaches the threshold (none if never),
+//   * OR in the block holding original key 0 (optional) and the row's own segment,
+//   * emit the dense byte masks and the ascending list of key blocks the attention
+//     kernel has to visit (own-segment blocks whose every key lies after the last
+//     query of the row are dropped from the list: they are fully masked).
+#include "pbs_common.h"
+#include <float.h>
+
+namespace {
+
+struct SelectArgs {
+  const float* P;          // (rows, nb, nb) or null when threshold_is_int_one
+  const float* thr_rows;   // per-head thresholds (rows) or null
+  float thr;
+  int thr_is_int_one;
+  int force_first;
+  const int32_t* idx;      // (rows, nb*bs)
+  int32_t* first_blk;      // (rows) workspace
+  int nb, bs, bps, S, n_pow2;
+  uint8_t* sel_mask;       // (rows, nb, nb) or null: selected | first-token
+  uint8_t* final_mask;     // (rows, nb, nb) or null: sel | own segment
+  int32_t* csr_cols;       // (rows, nb, nb) or null
+  int32_t* csr_cnt;        // (rows, nb)
+};
+
+__global__ __launch_bounds__(1024) void first_token_block_kernel(const int32_t* idx, int32_t* first_blk, int S_pad, int bs) {
+  __shared__ int found;
+  if (threadIdx.x == 0) found = -1;
+  __syncthreads();
+  const int32_t* row = idx + (int64_t)blockIdx.x * S_pad;
+  for (int i = threadIdx.x; i < S_pad; i += blockDim.x)
+    if (row[i] == 0) atomicMax(&found, i / bs);
+  __syncthreads();
+  if (threadIdx.x == 0) first_blk[blockIdx.x] = found;
+}
+
+__global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
+  extern __shared__ uint64_t keys[];
+  uint8_t* flag = reinterpret_cast<uint8_t*>(keys + a.n_pow2);
+  __shared__ int s_first;
+  __shared__ int s_min[256];
+  __shared__ int s_scan[256];
+  const int qb = blockIdx.x, row = blockIdx.y;
+  const int nb = a.nb;
+  const int seg_first = (qb / a.bps) * a.bps;
+  const int seg_end = min(seg_first + a.bps, nb);
+  const int64_t row_off = ((int64_t)row * nb + qb) * nb;
+
+  for (int kb = threadIdx.x; kb < nb; kb += blockDim.x) flag[kb] = 0;
+  s_min[threadIdx.x] = INT_MAX;
+
+  if (a.thr_is_int_one) {
+    __syncthreads();
+    for (int kb = threadIdx.x; kb < seg_first; kb += blockDim.x) flag[kb] = 1;
+  } else {
+    const float* p = a.P + row_off;
+    for (int i = threadIdx.x; i < a.n_pow2; i += blockDim.x) {
+      uint64_t key = ~0ull;
+      if (i < nb) {
+        float v = p[i];
+        if (v != v) v = 0.f;
+        else if (v == INFINITY) v = FLT_MAX;
+        else if (v == -INFINITY) v = -FLT_MAX;
+        key = desc_stable_key(v, (uint32_t)i);
+      }
+      keys[i] = key;
+    }
+    bitonic_sort_lds(keys, a.n_pow2);
+    if (threadIdx.x == 0) {
+      const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
+      double c = 0.0;
+      int first = -1;
+      for (int r = 0; r < nb; ++r) {
+        const float v = desc_key_value(keys[r]);
+        c += (double)v;
+        if ((float)c >= thr) {
+          first = r;
+          break;
+        }
+        if (v == 0.f) break;  // sorted: nothing positive follows, the sum cannot grow
+      }
+      s_first = first;
+    }
+    __syncthreads();
+    const int first = s_first;
+    for (int r = threadIdx.x; r <= first; r += blockDim.x) flag[(uint32_t)keys[r]] = 1;
+  }
+  __syncthreads();
+  if (a.force_first && threadIdx.x == 0) {
+    const int fb = a.first_blk[row];
+    if (fb >= 0 && fb < nb) flag[fb] = 1;
+  }
+  // smallest original key position of each own-segment block
+  for (int o = seg_first; o < seg_end; ++o) {
+    if (threadIdx.x < a.bs) {
+      const int v = a.idx[(int64_t)row * nb * a.bs + (int64_t)o * a.bs + threadIdx.x];
+      atomicMin(&s_min[o - seg_first], v);
+    }
+  }
+  __syncthreads();
+
+  const int q_last = min(qb * a.bs + a.bs - 1, a.S - 1);
+  const int per = (nb + 255) / 256;
+  const int k0 = threadIdx.x * per, k1 = min(k0 + per, nb);
+  int cnt = 0;
+  for (int kb = k0; kb < k1; ++kb) {
+    const bool own = kb >= seg_first && kb < seg_end;
+    const uint8_t s = flag[kb];
+    if (a.sel_mask) a.sel_mask[row_off + kb] = s;
+    if (a.final_mask) a.final_mask[row_off + kb] = s | (own ? 1 : 0);
+    const bool visit = own ? (s_min[kb - seg_first] <= q_last) : (s && kb < seg_first);
+    cnt += visit ? 1 : 0;
+  }
+  s_scan[threadIdx.x] = cnt;
+  __syncthreads();
+  for (int off = 1; off < 256; off <<= 1) {
+    int v = 0;
+    if ((int)threadIdx.x >= off) v = s_scan[threadIdx.x - off];
+    __syncthreads();
+    s_scan[threadIdx.x] += v;
+    __syncthreads();
+  }
+  int w = s_scan[threadIdx.x] - cnt;
+  if (a.csr_cols) {
+    for (int kb = k0; kb < k1; ++kb) {
+      const bool own = kb >= seg_first && kb < seg_end;
+      const bool visit = own ? (s_min[kb - seg_first] <= q_last) : (flag[kb] && kb < seg_first);
+      if (visit) a.csr_cols[row_off + w++] = kb;
+    }
+  }
+  if (threadIdx.x == 255) a.csr_cnt[(int64_t)row * nb + qb] = s_scan[255];
+}
+
+}  // namespace
+
+extern "C" size_t pbs_select_blocks_workspace_bytes(int rows) { return (size_t)rows * sizeof(int32_t); }
+
+extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
+                                 int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices,
+                                 int rows, int S, int block_size, int segment_size, uint8_t* sel_mask,
+                                 uint8_t* final_mask, int32_t* csr_cols, int32_t* csr_cnt, void* workspace,
+                                 size_t workspace_bytes, void* stream) {
+  PBS_REQUIRE(key_indices && csr_cnt, "pbs_select_blocks: null index / count pointer");
+  PBS_REQUIRE(threshold_is_int_one || block_attn_scores, "pbs_select_blocks: null score pointer");
+  PBS_REQUIRE(rows > 0 && rows <= 65535 && S > 0, "pbs_select_blocks: bad shape");
+  PBS_REQUIRE(block_size > 0 && block_size <= 256, "pbs_select_blocks: block_size %d outside (0, 256]", block_size);
+  PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_select_blocks: segment_size must be a multiple of block_size");
+  const int nb = (S + block_size - 1) / block_size;
+  const int bps = segment_size / block_size;
+  PBS_REQUIRE(bps <= 256, "pbs_select_blocks: more than 256 blocks per segment");
+  PBS_REQUIRE(nb <= 4096, "pbs_select_blocks: more than 4096 blocks per sequence (%d)", nb);
+  PBS_REQUIRE(workspace && workspace_bytes >= pbs_select_blocks_workspace_bytes(rows), "pbs_select_blocks: workspace too small");
+  SelectArgs a;
+  a.P = block_attn_scores; a.thr_rows = threshold_per_row; a.thr = threshold;
+  a.thr_is_int_one = threshold_is_int_one; a.force_first = force_select_first_block;
+  a.idx = key_indices; a.first_blk = (int32_t*)workspace;
+  a.nb = nb; a.bs = block_size; a.bps = bps; a.S = S; a.n_pow2 = next_pow2_int(nb);
+  a.sel_mask = sel_mask; a.final_mask = final_mask; a.csr_cols = csr_cols; a.csr_cnt = csr_cnt;
+  hipStream_t st = (hipStream_t)stream;
+  if (force_select_first_block)
+    hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size);
+  const size_t lds = (size_t)a.n_pow2 * sizeof(uint64_t) + (size_t)((nb + 15) / 16) * 16;
+  hipLaunchKernelGGL(select_blocks_kernel, dim3(nb, rows), dim3(256), lds, st, a);
+  return pbs_check_launch("pbs_select_blocks");
+}

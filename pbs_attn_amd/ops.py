@@ -1,0 +1,177 @@
+"""Stage-level torch wrappers over the C ABI (device pointers, strides, current
+stream).  Tensors are bf16, head_dim 128, block_size 128; all outputs are
+allocated through torch's caching allocator."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import _lib
+
+BLOCK = 128
+HEAD_DIM = 128
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return t.data_ptr() if t is not None else None
+
+
+def _rows16(t: torch.Tensor) -> torch.Tensor:
+    """Kernels need unit stride on head_dim and 16-byte aligned rows."""
+    if t.stride(-1) != 1 or any(s % 8 for s in t.stride()[:-1]) or t.data_ptr() % 16:
+        t = t.contiguous()
+    return t
+
+
+def _check_bf16_cuda(*ts):
+    for t in ts:
+        if not t.is_cuda:
+            raise _lib.PbsHipError("PBS HIP kernels need tensors on the GPU (there is no CPU path)")
+        if t.dtype != torch.bfloat16:
+            raise _lib.PbsHipError(f"PBS HIP kernels are bf16 only, got {t.dtype}")
+
+
+def score_keys(q, k, block_size, segment_size):
+    """(B, Hq, Sc) float32 key scores; permute_states.py:44-50."""
+    _check_bf16_cuda(q, k)
+    lib = _lib.load()
+    q, k = _rows16(q), _rows16(k)
+    B, Hq, S, D = q.shape
+    Hkv = k.shape[1]
+    Sc = (S // segment_size) * segment_size
+    scores = torch.empty((B, Hq, Sc), dtype=torch.float32, device=q.device)
+    ws_bytes = lib.pbs_score_keys_workspace_bytes(B, Hq, S, segment_size)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.pbs_score_keys(_ptr(q), _ptr(k), _ptr(scores), B, Hq, Hkv, S, D, block_size, segment_size,
+                                  q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                                  _ptr(ws), ws.numel(), _stream()), "pbs_score_keys")
+    return scores
+
+
+def segment_argsort(scores, seq_len, segment_size, block_size=BLOCK):
+    """scores (B, H, Sc) float32 -> int32 key indices (B, H, S_pad), S_pad = S rounded
+    up to the block; permute_states.py:56,71-81."""
+    lib = _lib.load()
+    B, H = scores.shape[:2]
+    scores = scores.contiguous().float()
+    s_pad = (seq_len + block_size - 1) // block_size * block_size
+    idx = torch.empty((B, H, s_pad), dtype=torch.int32, device=scores.device)
+    _lib.check(lib.pbs_segment_argsort(_ptr(scores), _ptr(idx), B * H, seq_len, s_pad, segment_size, _stream()),
+               "pbs_segment_argsort")
+    return idx
+
+
+def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean"):
+    """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128), pooled_k (B, Hq, nb, D)."""
+    _check_bf16_cuda(k, v)
+    if key_pool_mode not in ("mean", "max"):
+        raise ValueError(f"Invalid key_pool_mode: {key_pool_mode}")
+    lib = _lib.load()
+    k, v = _rows16(k), _rows16(v)
+    B, Hkv, S, D = k.shape
+    Hq = num_q_heads
+    nb = (S + BLOCK - 1) // BLOCK
+    assert idx.shape == (B, Hq, nb * BLOCK) and idx.dtype == torch.int32 and idx.is_contiguous()
+    perm_k = torch.empty((B, Hq, nb * BLOCK, D), dtype=k.dtype, device=k.device)
+    perm_vt = torch.empty((B, Hq, nb, D, BLOCK), dtype=k.dtype, device=k.device)
+    pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device)
+    _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k),
+                                 B, Hq, Hkv, S, D, BLOCK, k.stride(0), k.stride(1), k.stride(2),
+                                 v.stride(0), v.stride(1), v.stride(2), int(key_pool_mode == "max"), _stream()),
+               "pbs_gather_kv")
+    return perm_k, perm_vt, pooled_k
+
+
+def pool_q(q, query_pool_mode="mean"):
+    _check_bf16_cuda(q)
+    if query_pool_mode not in ("mean", "max"):
+        raise ValueError(f"Invalid query_pool_mode: {query_pool_mode}")
+    lib = _lib.load()
+    q = _rows16(q)
+    B, Hq, S, D = q.shape
+    nb = (S + BLOCK - 1) // BLOCK
+    pooled = torch.empty((B, Hq, nb, D), dtype=q.dtype, device=q.device)
+    _lib.check(lib.pbs_pool_q(_ptr(q), _ptr(pooled), B, Hq, S, D, BLOCK, q.stride(0), q.stride(1), q.stride(2),
+                              int(query_pool_mode == "max"), _stream()), "pbs_pool_q")
+    return pooled
+
+
+def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment):
+    """(B, H, nb, nb) float32 block probabilities; utils.py:30-33."""
+    _check_bf16_cuda(pooled_q, pooled_k)
+    lib = _lib.load()
+    pooled_q, pooled_k = pooled_q.contiguous(), pooled_k.contiguous()
+    B, H, nb, D = pooled_q.shape
+    P = torch.empty((B, H, nb, nb), dtype=torch.float32, device=pooled_q.device)
+    _lib.check(lib.pbs_block_logits_softmax(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D,
+                                            blocks_per_segment, _stream()), "pbs_block_logits_softmax")
+    return P
+
+
+def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segment_size,
+                  force_select_first_block=True, want_masks=True, want_csr=True, rows_shape=None):
+    """Returns (sel_mask, final_mask, csr_cols, csr_cnt).  ``threshold`` may be a
+    python float, the python int 1 (all candidates) or a (B, H) tensor."""
+    lib = _lib.load()
+    B, H = idx.shape[:2]
+    dev = idx.device
+    nb = (seq_len + block_size - 1) // block_size
+    is_int_one = isinstance(threshold, int) and not isinstance(threshold, bool) and threshold == 1
+    thr_rows = None
+    thr = 0.0
+    if isinstance(threshold, torch.Tensor):
+        thr_rows = threshold.to(device=dev, dtype=torch.float32).expand(B, H).contiguous()
+    elif not is_int_one:
+        thr = float(threshold)
+    P = None
+    if not is_int_one:
+        P = block_attn_scores.contiguous()
+        assert P.dtype == torch.float32 and P.shape == (B, H, nb, nb)
+    sel = torch.empty((B, H, nb, nb), dtype=torch.bool, device=dev) if want_masks else None
+    fin = torch.empty((B, H, nb, nb), dtype=torch.bool, device=dev) if want_masks else None
+    cols = torch.empty((B, H, nb, nb), dtype=torch.int32, device=dev) if want_csr else None
+    cnt = torch.empty((B, H, nb), dtype=torch.int32, device=dev)
+    ws = torch.empty(max(lib.pbs_select_blocks_workspace_bytes(B * H), 16), dtype=torch.uint8, device=dev)
+    _lib.check(lib.pbs_select_blocks(_ptr(P), _ptr(thr_rows), thr, int(is_int_one), int(bool(force_select_first_block)),
+                                     _ptr(idx), B * H, seq_len, block_size, segment_size, _ptr(sel), _ptr(fin),
+                                     _ptr(cols), _ptr(cnt), _ptr(ws), ws.numel(), _stream()), "pbs_select_blocks")
+    return sel, fin, cols, cnt
+
+
+def sparse_attn_fwd(q, perm_k, perm_vt, idx, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
+    _check_bf16_cuda(q, perm_k, perm_vt)
+    lib = _lib.load()
+    q = _rows16(q)
+    B, Hq, S, D = q.shape
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    if out is None:
+        out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
+    assert perm_k.is_contiguous() and perm_vt.is_contiguous() and idx.is_contiguous()
+    assert csr_cols.is_contiguous() and csr_cnt.is_contiguous()
+    _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(idx), _ptr(csr_cols), _ptr(csr_cnt),
+                                       _ptr(out), B, Hq, S, D, BLOCK, segment_size,
+                                       q.stride(0), q.stride(1), q.stride(2),
+                                       out.stride(0), out.stride(1), out.stride(2), softmax_scale, _stream()),
+               "pbs_sparse_attn_fwd")
+    return out
+
+
+def unpermute(o_perm, q_idx=None, out=None):
+    """out[b, h, q_idx[b, h, i]] = o_perm[b, h, i]; identity (no launch) when the
+    queries were not permuted."""
+    lib = _lib.load()
+    if q_idx is None and out is None:
+        out = o_perm
+    o_perm = o_perm if (q_idx is None and out is o_perm) else o_perm.contiguous()
+    if out is None:
+        out = torch.empty_like(o_perm)
+    B, H, S, D = o_perm.shape
+    _lib.check(lib.pbs_unpermute(_ptr(o_perm), _ptr(q_idx), _ptr(out), B, H, S, D,
+                                 out.stride(0), out.stride(1), out.stride(2), _stream()), "pbs_unpermute")
+    return out

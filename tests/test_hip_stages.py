@@ -1,0 +1,316 @@
+"""GPU parity of every HIP stage against the CPU oracle, through the C ABI.
+
+Index and mask stages are compared bit-exactly on identical score tensors;
+floating-point stages within stated tolerances."""
+import math
+
+import pytest
+import torch
+
+from oracle import pbs_oracle as O
+from pbs_attn_amd import ops
+from pbs_attn_amd import pbs as P
+from tests.util import assert_attn_close, expand_kv, quantised_scores, small_case
+
+pytestmark = pytest.mark.gpu
+
+
+# ---------------------------------------------------------------- key scores
+@pytest.mark.parametrize("Hq,Hkv,S,seg", [(4, 2, 1024, 256), (2, 2, 1408, 512), (7, 1, 2048, 1024)])
+def test_score_keys_matches_oracle(dev, Hq, Hkv, S, seg):
+    q, k, _ = small_case(1, Hq, Hkv, S, seed=3)
+    ref = O.key_scores(q, k, 128, seg)
+    got = ops.score_keys(q.to(dev), k.to(dev), 128, seg).cpu()
+    assert got.shape == ref.shape
+    # probabilities sum to one over the scored keys
+    assert torch.allclose(got.sum(-1), torch.ones_like(got.sum(-1)), atol=2e-3)
+    rel = (got - ref).abs() / ref.abs().clamp_min(1e-12)
+    # logits are bf16 values: a one-ulp flip of a logit moves its probability by < 1 %
+    assert rel.max().item() < 3e-2, rel.max().item()
+    assert rel.mean().item() < 2e-3, rel.mean().item()
+
+
+def test_score_keys_strided_query(dev):
+    # Q as the patched forward hands it over: (B, S, H, D) memory viewed as (B, H, S, D)
+    q, k, _ = small_case(2, 4, 2, 768, seed=5)
+    qd = q.to(dev).transpose(1, 2).contiguous().transpose(1, 2)
+    assert not qd.is_contiguous()
+    a = ops.score_keys(qd, k.to(dev), 128, 256)
+    b = ops.score_keys(q.to(dev), k.to(dev), 128, 256)
+    assert torch.equal(a, b)
+
+
+# ---------------------------------------------------------------- segment sort
+@pytest.mark.parametrize("S,seg", [(1024, 256), (4096, 1024), (1000, 256), (1536, 384), (700, 512), (2048, 128)])
+def test_segment_argsort_bit_exact_with_ties(dev, S, seg):
+    B, H = 2, 3
+    sc = (S // seg) * seg
+    scores = quantised_scores((B, H, sc), levels=37, seed=S + seg)
+    ref = O.segment_argsort(scores, S, seg)
+    got = ops.segment_argsort(scores.to(dev), S, seg).cpu()
+    s_pad = (S + 127) // 128 * 128
+    assert got.shape == (B, H, s_pad)
+    assert torch.equal(got[:, :, :S].long(), ref)
+    assert torch.equal(got[:, :, S:].long(), torch.arange(S, s_pad).expand(B, H, -1))
+
+
+def test_segment_argsort_special_values(dev):
+    scores = torch.tensor([0.0, -0.0, 1.0, float("inf"), 1.0, 1e-45, -1.0, 0.0] * 16).view(1, 1, 128)
+    ref = O.segment_argsort(scores, 128, 128)
+    got = ops.segment_argsort(scores.to(dev), 128, 128).cpu()
+    assert torch.equal(got.long(), ref)
+
+
+# ---------------------------------------------------------------- gather + pooling
+@pytest.mark.parametrize("Hq,Hkv,S,mode", [(4, 2, 1024, "mean"), (4, 4, 900, "mean"), (7, 1, 512, "max")])
+def test_gather_kv_bitwise(dev, Hq, Hkv, S, mode):
+    q, k, v = small_case(2, Hq, Hkv, S, seed=7)
+    g = torch.Generator().manual_seed(11)
+    seg = 256
+    sc = (S // seg) * seg
+    idx = O.segment_argsort(torch.rand((2, Hq, sc), generator=g), S, seg)
+    s_pad = (S + 127) // 128 * 128
+    idx_pad = torch.cat([idx, torch.arange(S, s_pad).expand(2, Hq, -1)], -1).int()
+    perm_k, perm_vt, pooled_k = ops.gather_kv(k.to(dev), v.to(dev), idx_pad.to(dev), Hq, mode)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref_k, ref_v = O.gather_rows(ke, idx), O.gather_rows(ve, idx)
+    assert torch.equal(perm_k.cpu()[:, :, :S], ref_k)
+    assert (perm_k.cpu()[:, :, S:] == 0).all()
+    nb = s_pad // 128
+    got_v = perm_vt.cpu().transpose(-1, -2).reshape(2, Hq, s_pad, 128)
+    assert torch.equal(got_v[:, :, :S], ref_v)
+    assert (got_v[:, :, S:] == 0).all()
+    pk_pad, _ = O.pad_to_block(ref_k, idx, 128)
+    ref_pool = O.pool_blocks(pk_pad, 128, mode)
+    if mode == "max":
+        assert torch.equal(pooled_k.cpu(), ref_pool)
+    else:
+        assert torch.allclose(pooled_k.cpu().float(), ref_pool.float(), atol=1e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("mode", ["mean", "max"])
+def test_pool_q(dev, mode):
+    q, _, _ = small_case(2, 3, 3, 900, seed=9)
+    qp, _ = O.pad_to_block(q, torch.arange(900).expand(2, 3, -1), 128)
+    ref = O.pool_blocks(qp, 128, mode)
+    got = ops.pool_q(q.to(dev), mode).cpu()
+    if mode == "max":
+        assert torch.equal(got, ref)
+    else:
+        assert torch.allclose(got.float(), ref.float(), atol=1e-3, rtol=1e-2)
+
+
+# ---------------------------------------------------------------- block logits softmax
+@pytest.mark.parametrize("nb,bps", [(8, 2), (40, 8), (33, 1), (64, 64)])
+def test_block_logits_softmax(dev, nb, bps):
+    g = torch.Generator().manual_seed(nb)
+    pq = (torch.randn((2, 3, nb, 128), generator=g) * 2).bfloat16()
+    pk = (torch.randn((2, 3, nb, 128), generator=g) * 2).bfloat16()
+    cand, _ = O.candidate_masks(nb, bps)
+    ref = O.block_logits_softmax(pq, pk, cand)
+    got = ops.block_logits_softmax(pq.to(dev), pk.to(dev), bps).cpu()
+    assert torch.equal(torch.isnan(got), torch.isnan(ref))
+    ok = ~torch.isnan(ref)
+    assert torch.equal(got[ok] == 0, ref[ok] == 0)
+    assert torch.allclose(got[ok], ref[ok], rtol=3e-2, atol=1e-6)
+
+
+# ---------------------------------------------------------------- selection
+def _oracle_selection(P_scores, thr, idx_pad, nb, bps, force_first):
+    is_one = isinstance(thr, int) and thr == 1
+    cand, segm = O.candidate_masks(nb, bps)
+    if is_one:
+        sel = cand.view(1, 1, nb, nb).expand(P_scores.shape).clone()
+    else:
+        sel = O.select_blocks(P_scores, thr)
+    if force_first:
+        sel = sel | O.first_token_mask(idx_pad.long(), 128)
+    return sel, sel | segm[None, None]
+
+
+@pytest.mark.parametrize("nb,bps,thr,force_first", [
+    (8, 2, 0.9, True), (32, 2, 0.8, True), (32, 8, 0.95, False), (40, 8, 1.0, True), (40, 8, 1, True),
+    (33, 1, 0.5, True), (100, 4, 0.0, True), (64, 2, "tensor", True)])
+def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
+    B, H, S = 2, 3, nb * 128 - 5
+    g = torch.Generator().manual_seed(nb * 7 + bps)
+    cand, _ = O.candidate_masks(nb, bps)
+    # bf16-valued logits -> many exactly equal probabilities, as in the real path
+    logits = (torch.randn((B, H, nb, nb), generator=g) * 1.5).bfloat16().float()
+    Pm = torch.softmax(logits.masked_fill(~cand, float("-inf")), -1)
+    if thr == "tensor":
+        thr = torch.rand((B, H), generator=g) * 0.5 + 0.45
+    seg = bps * 128
+    sc = (S // seg) * seg
+    idx = O.segment_argsort(torch.rand((B, H, sc), generator=g), S, seg) if sc else torch.arange(S).expand(B, H, -1)
+    idx_pad = torch.cat([idx, torch.arange(S, nb * 128).expand(B, H, -1)], -1).int()
+    ref_sel, ref_fin = _oracle_selection(Pm, thr, idx_pad, nb, bps, force_first)
+    thr_dev = thr.to(dev) if isinstance(thr, torch.Tensor) else thr
+    sel, fin, cols, cnt = ops.select_blocks(Pm.to(dev), thr_dev, idx_pad.to(dev), S, 128, seg, force_first)
+    assert torch.equal(sel.cpu(), ref_sel)
+    assert torch.equal(fin.cpu(), ref_fin)
+    # the visit list = final mask restricted to segments not after the query block's,
+    # minus own-segment blocks whose every key lies after the block's last query
+    cols, cnt = cols.cpu(), cnt.cpu()
+    qseg = torch.arange(nb) // bps
+    kmin = idx_pad.view(B, H, nb, 128).min(-1).values
+    for b in range(B):
+        for h in range(H):
+            for qb in range(nb):
+                q_last = min(qb * 128 + 127, S - 1)
+                want = [kb for kb in range(nb) if ref_fin[b, h, qb, kb] and qseg[kb] <= qseg[qb]
+                        and not (qseg[kb] == qseg[qb] and kmin[b, h, kb] > q_last)]
+                assert cols[b, h, qb, :cnt[b, h, qb]].tolist() == want
+
+
+def test_select_blocks_nan_rows_and_zero_rows(dev):
+    nb, bps = 16, 4
+    Pm = torch.zeros((1, 2, nb, nb))
+    Pm[:, :, :4] = float("nan")
+    Pm[0, 1, 9, :8] = 0.125
+    idx_pad = torch.arange(nb * 128).expand(1, 2, -1).int()
+    ref_sel, ref_fin = _oracle_selection(Pm, 0.9, idx_pad, nb, bps, False)
+    sel, fin, _, _ = ops.select_blocks(Pm.to(dev), 0.9, idx_pad.to(dev), nb * 128, 128, bps * 128, False)
+    assert torch.equal(sel.cpu(), ref_sel) and torch.equal(fin.cpu(), ref_fin)
+    assert ref_sel[0, 0].sum() == 0 and ref_sel[0, 1, 9].sum() == 8
+
+
+# ---------------------------------------------------------------- sparse attention
+def _run_attention_case(dev, B, Hq, Hkv, S, seg, thr, seed):
+    q, k, v = small_case(B, Hq, Hkv, S, seed=seed)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    out_ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, seg, thr, return_intermediates=True)
+    idx = mid["key_indices"]
+    nb = (S + 127) // 128
+    idx_pad = torch.cat([idx, torch.arange(S, nb * 128).expand(B, Hq, -1)], -1).int().contiguous().to(dev)
+    # same indices and same block probabilities as the oracle -> same masks (asserted), then attention
+    perm_k, perm_vt, _ = ops.gather_kv(k.to(dev), v.to(dev), idx_pad, Hq)
+    sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), thr, idx_pad, S, 128, seg, True)
+    assert torch.equal(fin.cpu(), mid["final_mask"])
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, idx_pad, cols, cnt, seg).cpu()
+    dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], idx, mid["final_mask"], 128)
+    assert_attn_close(out, out_ref, what="HIP vs oracle naive path")
+    assert_attn_close(out, dense, what="HIP vs dense fp32 oracle")
+    assert_attn_close(out_ref, dense, what="oracle naive vs dense fp32 oracle")
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,seg,thr", [
+    (1, 4, 2, 1024, 256, 0.9), (2, 2, 2, 1536, 512, 0.8), (1, 7, 1, 1024, 256, 0.95),
+    (1, 2, 1, 1000, 256, 0.9), (1, 2, 2, 1300, 512, 0.9), (1, 2, 2, 1024, 128, 0.9), (1, 2, 1, 1024, 256, 1)])
+def test_sparse_attention_given_oracle_masks(dev, B, Hq, Hkv, S, seg, thr):
+    _run_attention_case(dev, B, Hq, Hkv, S, seg, thr, seed=S + seg)
+
+
+def test_sparse_attention_strided_query(dev):
+    # Q in the (B, S, H, D) memory layout the patched forward produces: same bits as contiguous Q
+    q, k, v = small_case(2, 4, 2, 768, seed=21)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    perm = P.apply_permutation(qd, kd, vd, 128, 256)
+    sel = P.permuted_block_selection(qd, perm, 128, 256, 0.9)
+    args = (perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], 256)
+    q_strided = qd.transpose(1, 2).contiguous().transpose(1, 2)
+    assert not q_strided.is_contiguous()
+    out_c = ops.sparse_attn_fwd(qd, *args)
+    out_s = ops.sparse_attn_fwd(q_strided, *args)
+    assert torch.equal(out_c, out_s)
+    # and into a strided output buffer
+    buf = torch.empty((2, 768, 4, 128), dtype=q.dtype, device=dev).transpose(1, 2)
+    ops.sparse_attn_fwd(q_strided, *args, out=buf)
+    assert torch.equal(buf, out_c)
+
+
+# ---------------------------------------------------------------- whole pipeline on the GPU
+def _pipeline_vs_dense(dev, q, k, v, seg, thr, **kw):
+    """Runs every HIP stage; checks the output against the dense fp32 oracle applied to
+    the HIP path's own indices and mask, and the indices / masks for self-consistency."""
+    B, Hq, S, D = q.shape
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    perm = P.apply_permutation(qd, kd, vd, 128, seg)
+    sel = P.permuted_block_selection(qd, perm, 128, seg, thr, **kw)
+    out = ops.sparse_attn_fwd(qd, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+    idx = perm.key_indices.cpu()[:, :, :S].long()
+    # permutation stays inside segments
+    sc = (S // seg) * seg
+    srt = idx[:, :, :sc].view(B, Hq, -1, seg).sort(-1).values
+    assert torch.equal(srt, torch.arange(sc).view(1, 1, -1, seg).expand_as(srt))
+    assert torch.equal(idx[:, :, sc:], torch.arange(sc, S).expand(B, Hq, -1))
+    pk = perm.permuted_keys().cpu()
+    pv = perm.permuted_values().cpu()
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    assert torch.equal(pk, O.gather_rows(ke, idx)) and torch.equal(pv, O.gather_rows(ve, idx))
+    dense = O.dense_masked_attention_fp32(q, pk, pv, idx, sel["final_mask"].cpu(), 128)
+    assert_attn_close(out.cpu(), dense, what="HIP pipeline vs dense fp32 oracle on its own mask")
+    return out, perm, sel
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,seg,thr", [
+    (1, 4, 2, 2048, 256, 0.9), (2, 7, 1, 1024, 256, 0.9), (1, 2, 2, 1900, 512, 0.8), (1, 4, 4, 4096, 1024, 0.95)])
+def test_pipeline_against_dense_oracle(dev, B, Hq, Hkv, S, seg, thr):
+    q, k, v = small_case(B, Hq, Hkv, S, seed=S)
+    _pipeline_vs_dense(dev, q, k, v, seg, thr)
+
+
+def test_pipeline_sorted_scores_are_non_increasing(dev):
+    q, k, v = small_case(1, 4, 2, 2048, seed=2)
+    qd, kd = q.to(dev), k.to(dev)
+    scores = ops.score_keys(qd, kd, 128, 256)
+    idx = ops.segment_argsort(scores, 2048, 256)
+    g = torch.gather(scores, 2, idx[:, :, :2048].long()).view(1, 4, -1, 256)
+    assert (g[..., 1:] <= g[..., :-1]).all()
+    # and bit-exact with the oracle's sort of the very same score tensor
+    assert torch.equal(idx.cpu().long(), O.segment_argsort(scores.cpu(), 2048, 256))
+
+
+@pytest.mark.parametrize("S,seg", [(2048, 256), (1111, 256), (1024, 1024), (300, 1024), (128, 256), (77, 256)])
+def test_threshold_int_one_equals_dense_causal(dev, S, seg):
+    # known answer: with every candidate selected the result is plain causal attention,
+    # whatever the permutation; S <= segment takes the no-permutation route
+    q, k, v = small_case(1, 4, 2, S, seed=S)
+    fwd = P.permuted_block_sparse_attn_fwd
+    out = fwd(q.to(dev), k.to(dev), v.to(dev), 128, seg, 1, True).cpu()
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), ke.float(), ve.float(), is_causal=True)
+    assert_attn_close(out, ref, what="threshold=1 vs SDPA")
+
+
+def test_ones_value_rows_sum_to_one(dev):
+    # V = 1 everywhere: any normalised attention returns exactly ones
+    q, k, v = small_case(1, 2, 2, 1536, seed=4)
+    out = P.permuted_block_sparse_attn_fwd(q.to(dev), k.to(dev), torch.ones_like(v).to(dev), 128, 256, 0.9, True)
+    assert torch.allclose(out.float().cpu(), torch.ones(1, 2, 1536, 128), atol=8e-3)
+
+
+def test_end_to_end_matches_oracle_when_selection_agrees(dev):
+    # full HIP pipeline vs full oracle pipeline; they can only differ where a score
+    # near-tie flips the permutation, so compare where both chose the same key order
+    q, k, v = small_case(1, 4, 2, 2048, seed=12)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, 256, 0.9, return_intermediates=True)
+    out = P.permuted_block_sparse_attn_fwd(q.to(dev), k.to(dev), v.to(dev), 128, 256, 0.9, True).cpu()
+    diff = (out.float() - ref.float()).abs()
+    # thresholded selection drops ~10 % of the mass: different but equally valid selections
+    # still agree to that order; identical selections agree to bf16 tolerance
+    assert diff.mean().item() < 2e-2
+    assert torch.isfinite(out.float()).all()
+
+
+def test_inputs_not_mutated_and_output_fresh(dev):
+    q, k, v = small_case(1, 2, 2, 512, seed=6)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    q0, k0, v0 = qd.clone(), kd.clone(), vd.clone()
+    out = P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 256, 0.9, True)
+    assert torch.equal(qd, q0) and torch.equal(kd, k0) and torch.equal(vd, v0)
+    assert out.shape == q.shape and out.dtype == q.dtype and out.data_ptr() != qd.data_ptr()
+
+
+def test_error_behaviour(dev):
+    q, k, v = small_case(1, 2, 2, 512, seed=6)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    with pytest.raises(AssertionError):
+        P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 256, 0.9, False)
+    with pytest.raises(AssertionError):
+        P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 200, 0.9, True)
+    with pytest.raises(ValueError):
+        P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 256, 0.9, True, query_pool_mode="median")
+    with pytest.raises(AssertionError):
+        P.permuted_block_sparse_attn_fwd(qd, kd[:, :, :256], vd[:, :, :256], 128, 256, 0.9, True)
