@@ -1,0 +1,249 @@
+#!/usr/bin/env python3
+"""PBS-Attn prefill-attention benchmark on one MI355X.
+
+A step = one full pass of the hot path (key scoring, segment sort, K/V gather,
+block estimation + selection, block-sparse attention, un-permutation) over one
+synthetic Llama-3.1-8B-shaped attention layer already resident in HBM.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
+
+prints ONE JSON line.  `value` is the effective TFLOP/s of the whole pass
+(4 * 128 * 128 * 128 FLOP per visited block pair / step time); `roofline` prices
+the dominant kernel (the block-sparse attention) against the bf16 dense MFMA peak
+with its duration taken from HIP events recorded around it inside the timed steps;
+`cpu_baseline` times the CPU restatement of the reference's torch path on a bounded
+sample on this host's cores.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+FLOP_PER_BLOCK_PAIR = 4.0 * 128 * 128 * 128
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+class StageTimer:
+    """Records a HIP event after every stage of every step on the launch stream."""
+
+    def __init__(self, torch):
+        self.torch = torch
+        self.steps = []
+
+    def begin(self):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.steps.append([("start", ev)])
+
+    def mark(self, name):
+        ev = self.torch.cuda.Event(enable_timing=True)
+        ev.record()
+        self.steps[-1].append((name, ev))
+
+    def summary(self):
+        tot = {}
+        for marks in self.steps:
+            for (_, e0), (name, e1) in zip(marks[:-1], marks[1:]):
+                tot.setdefault(name, []).append(e0.elapsed_time(e1))
+        return {k: sum(v) / len(v) for k, v in tot.items()}
+
+
+def cpu_baseline(cfg, q, k, v, seconds_budget=20.0):
+    """The reference's torch CPU path (restated in oracle/) on the SAME workload,
+    bounded to whole query heads: head after head until `seconds_budget` is spent
+    (at least one).  The rate is visited-block FLOPs per second of CPU time."""
+    import torch
+    from oracle import pbs_oracle as O
+    G = cfg["Hq"] // cfg["Hkv"]
+    flops, spent, heads = 0.0, 0.0, 0
+    for h in range(cfg["Hq"]):
+        qs = q[:1, h:h + 1].cpu()
+        ks, vs = k[:1, h // G:h // G + 1].cpu(), v[:1, h // G:h // G + 1].cpu()
+        t0 = time.perf_counter()
+        _, mid = O.permuted_block_sparse_attn_fwd(qs, ks, vs, cfg["block"], cfg["segment"], cfg["threshold"],
+                                                  return_intermediates=True)
+        spent += time.perf_counter() - t0
+        flops += O.visited_block_pairs(mid["final_mask"], cfg["segment"] // cfg["block"]) * FLOP_PER_BLOCK_PAIR
+        heads += 1
+        log(f"[bench] cpu baseline: head {h} done, {spent:.1f} s so far")
+        if spent > seconds_budget:
+            break
+    return {"value": flops / spent / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"oracle torch CPU path on {heads} of {cfg['B'] * cfg['Hq']} (batch, query head) slices of the "
+                      f"same workload (S={cfg['S']}, segment {cfg['segment']}, threshold {cfg['threshold']}), "
+                      f"{spent:.1f} s, os.cpu_count()={os.cpu_count()}",
+            "ms_per_head": spent / heads * 1e3}
+
+
+def dense_sdpa_ms(torch, q, k, v, reps=3):
+    """Dense causal flash attention of the torch ROCm wheel on the same tensors."""
+    F = torch.nn.functional
+    try:
+        from torch.nn.attention import SDPBackend, sdpa_kernel
+        ctx = lambda: sdpa_kernel([SDPBackend.FLASH_ATTENTION])  # noqa: E731
+        with ctx():
+            F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        with ctx():
+            for _ in range(reps):
+                F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / reps
+    except Exception as exc:  # the baseline is informative only
+        log(f"[bench] dense SDPA baseline unavailable: {type(exc).__name__}: {exc}")
+        return None
+
+
+def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=True):
+    from pbs_attn_amd import pbs as P
+    from pbs_attn_amd.synth import make_workload
+    dev = torch.device("cuda:0")
+    cfg, q, k, v = make_workload(name, seed=seed, device=dev, **(overrides or {}))
+    B, Hq, Hkv, S, D = cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["S"], cfg["D"]
+    bs, seg, thr = cfg["block"], cfg["segment"], cfg["threshold"]
+    nb = (S + bs - 1) // bs
+
+    def step():
+        return P.permuted_block_sparse_attn_fwd(q, k, v, bs, seg, thr, True)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    timer = StageTimer(torch)
+    P.stage_timer = timer
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        timer.begin()
+        out = step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / steps
+    P.stage_timer = None
+    stages = timer.summary()
+
+    # visited block pairs of this input (one extra selection pass, outside the timed region)
+    perm = P.apply_permutation(q, k, v, bs, seg)
+    sel = P.permuted_block_selection(q, perm, bs, seg, thr, want_masks=False)
+    n_vis = int(sel["csr_cnt"].sum().item())
+    causal_pairs = B * Hq * nb * (nb + 1) // 2
+    flops = n_vis * FLOP_PER_BLOCK_PAIR
+    attn_ms = stages["sparse_attn"]
+    res = {
+        "workload": name, "B": B, "Hq": Hq, "Hkv": Hkv, "S": S, "D": D, "block": bs, "segment": seg,
+        "threshold": thr, "generator": cfg["kind"], "seed": seed,
+        "ms_per_step": wall_ms, "stage_ms": stages, "visited_block_pairs": n_vis,
+        "density_vs_causal": n_vis / causal_pairs,
+        "effective_tflops_pipeline": flops / (wall_ms * 1e-3) / 1e12,
+        "effective_tflops_attn_kernel": flops / (attn_ms * 1e-3) / 1e12,
+        "dense_causal_flop": 4.0 * S * S * D / 2 * Hq * B,
+    }
+    # HBM-bound stages: algorithmic bytes / stage time
+    e = 2
+    score_b = B * Hkv * S * D * e + B * Hq * bs * D * e + B * Hq * S * 4
+    gather_b = 2 * B * Hkv * S * D * e + B * Hq * S * 4 + 2 * B * Hq * S * D * e
+    est_b = B * Hq * S * D * e + B * Hq * nb * nb * 4
+    res["hbm_gbs"] = {
+        "score": score_b / (stages["score"] * 1e-3) / 1e9 if "score" in stages else None,
+        "gather": gather_b / (stages["gather"] * 1e-3) / 1e9,
+        "estimate": est_b / (stages["estimate"] * 1e-3) / 1e9 if "estimate" in stages else None,
+    }
+    if with_dense:
+        res["dense_sdpa_ms"] = dense_sdpa_ms(torch, q, k, v)
+        # the build's own kernel on the full causal mask (every candidate selected, one block per segment)
+        for _ in range(2):
+            P.permuted_block_sparse_attn_fwd(q, k, v, bs, bs, 1, True)
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        P.permuted_block_sparse_attn_fwd(q, k, v, bs, bs, 1, True)
+        e1.record()
+        torch.cuda.synchronize()
+        res["dense_own_kernel_ms"] = e0.elapsed_time(e1)
+        if res["dense_sdpa_ms"]:
+            res["speedup_vs_dense_sdpa"] = res["dense_sdpa_ms"] / wall_ms
+    del out
+    return res, (cfg, q, k, v)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=5)
+    ap.add_argument("--warmup", type=int, default=2)
+    ap.add_argument("--workload", default="cfg2", help="cfg0 | cfg1 | cfg2 | cfg3 (see pbs_attn_amd/synth.py)")
+    ap.add_argument("--segment", type=int, default=None)
+    ap.add_argument("--threshold", type=float, default=None)
+    ap.add_argument("--kind", default=None, help="override the input generator, e.g. strong_heavy")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this path is measured on ONE GPU (it shards over heads with no exchange); "
+            "run with --gpus 1.")
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        log("bench.py: no GPU visible; the HIP path has no CPU fallback.")
+        sys.exit(1)
+    from pbs_attn_amd import _lib
+    _lib.load()
+
+    overrides = {}
+    if args.segment:
+        overrides["segment"] = args.segment
+    if args.threshold is not None:
+        overrides["threshold"] = args.threshold
+    if args.kind:
+        overrides["kind"] = args.kind
+    res, inputs = run_workload(torch, args.workload, args.steps, args.warmup, overrides=overrides,
+                               with_dense=not args.no_dense)
+    log("[bench] " + json.dumps(res))
+
+    attn_s = res["stage_ms"]["sparse_attn"] * 1e-3
+    achieved = res["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / attn_s / 1e12
+    line = {
+        "metric": "pbs_prefill_attn_effective_tflops",
+        "value": res["effective_tflops_pipeline"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": res["ms_per_step"],
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: Llama-3.1-8B attention layer B={res['B']} Hq={res['Hq']} "
+                               f"Hkv={res['Hkv']} D={res['D']} S={res['S']}, block {res['block']}, segment "
+                               f"{res['segment']}, threshold {res['threshold']}, generator {res['generator']} seed {res['seed']}",
+                   "density_vs_causal": res["density_vs_causal"],
+                   "visited_block_pairs": res["visited_block_pairs"]},
+        "roofline": {"bound": "mfma", "kernel": "sparse_attn_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
+                     "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS, "traffic": None,
+                     "kernel_ms": res["stage_ms"]["sparse_attn"]},
+        "stage_ms": res["stage_ms"],
+        "hbm_gbs": res["hbm_gbs"],
+        "dense_sdpa_ms": res.get("dense_sdpa_ms"),
+        "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
+        "speedup_vs_dense_sdpa": res.get("speedup_vs_dense_sdpa"),
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(*inputs, seconds_budget=args.cpu_seconds)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -27,6 +27,15 @@ from . import ops
 
 _warned_use_triton = False
 
+# Optional profiling hook: an object with ``mark(stage_name)``, called after each
+# stage has been enqueued (the benchmark records a HIP event there).
+stage_timer = None
+
+
+def _mark(name):
+    if stage_timer is not None:
+        stage_timer.mark(name)
+
 
 @dataclass
 class PermutedKV:
@@ -63,8 +72,11 @@ def apply_permutation(query_states, key_states, value_states, block_size, segmen
     else:
         if scores is None:
             scores = ops.score_keys(query_states, key_states, block_size, segment_size)
+            _mark("score")
         idx = ops.segment_argsort(scores, S, segment_size, block_size)
+        _mark("sort")
     perm_k, perm_vt, pooled_k = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode)
+    _mark("gather")
     return PermutedKV(idx, perm_k, perm_vt, pooled_k, S)
 
 
@@ -86,8 +98,10 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
     if P is None and (not is_int_one or want_masks):
         pooled_q = ops.pool_q(query_states, query_pool_mode)
         P = ops.block_logits_softmax(pooled_q, perm.pooled_k, segment_size // block_size)
+        _mark("estimate")
     sel, fin, cols, cnt = ops.select_blocks(P, threshold, perm.key_indices, S, block_size, segment_size,
                                             force_select_first_block, want_masks=want_masks)
+    _mark("select")
     return dict(block_attn_scores=P, block_mask=sel, final_mask=fin, csr_cols=cols, csr_cnt=cnt)
 
 
@@ -130,8 +144,11 @@ def permuted_block_sparse_attn_fwd(
                                    force_select_first_block, query_pool_mode, key_pool_mode, want_masks=False)
     out = ops.sparse_attn_fwd(query_states, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"],
                               sel["csr_cnt"], segment_size, 1.0 / math.sqrt(head_dim))
+    _mark("sparse_attn")
     # queries are not permuted (pbs.py:191-193): un-permutation is the identity
-    return ops.unpermute(out)
+    out = ops.unpermute(out)
+    _mark("unpermute")
+    return out
 
 
 # the patched Hugging Face forward may hand K/V over at the KV-head count
