@@ -1,0 +1,177 @@
+"""Host-side logic without a GPU: the C ABI exports what the header declares, the
+import paths and factory of the plug-in boundary, the Hugging Face patcher on tiny
+random-init models (with the CPU oracle standing in as prefill_fn), and that the
+product path refuses to run without the GPU."""
+import ctypes
+import os
+import re
+from functools import partial
+
+import pytest
+import torch
+
+from oracle import pbs_oracle as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "pbs_hip.h")
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pbs_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from pbs_attn_amd import _lib
+    if not os.path.exists(_lib.LIB_PATH):
+        from pbs_attn_amd.build import build_library
+        build_library()
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    names = _declared_symbols()
+    assert len(names) >= 12
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in include/pbs_hip.h but not exported"
+    assert set(names) == set(_lib.SIGNATURES), "ctypes signatures and header disagree"
+    assert _lib.load().pbs_abi_version() == 1
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    # argument validation happens before any launch: safe on a CPU-only host
+    rc = lib.pbs_segment_argsort(None, None, 1, 128, 128, 128, None)
+    assert rc < 0 and b"null" in lib.pbs_last_error()
+    rc = lib.pbs_pool_q(1, 1, 1, 1, 128, 64, 128, 0, 0, 0, 0, None)
+    assert rc < 0 and b"head_dim" in lib.pbs_last_error()
+    with pytest.raises(_lib.PbsHipError):
+        _lib.check(rc, "pbs_pool_q")
+
+
+def test_reference_import_paths():
+    from pbs_attn import permuted_block_sparse_attn_fwd as a
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill, get_permuted_block_sparse_attn_fwd
+    from pbs_attn.src.pbs import permuted_block_sparse_attn_fwd as b
+    assert a is b and callable(apply_patch_with_prefill) and callable(get_permuted_block_sparse_attn_fwd)
+
+
+def test_factory_defaults_and_introspection():
+    from pbs_attn.patch.huggingface import get_permuted_block_sparse_attn_fwd
+    fn = get_permuted_block_sparse_attn_fwd()
+    assert isinstance(fn, partial)
+    assert fn.func.__name__ == "permuted_block_sparse_attn_fwd"
+    assert fn.keywords == dict(block_size=128, segment_size=256, threshold=0.9, causal=True,
+                               force_select_first_block=True, use_triton=True, query_pool_mode="mean",
+                               key_pool_mode="mean")
+    names = fn.func.__code__.co_varnames[:fn.func.__code__.co_argcount]
+    assert names == ("query_states", "key_states", "value_states", "block_size", "segment_size", "threshold",
+                     "causal", "force_select_first_block", "use_triton", "query_pool_mode", "key_pool_mode")
+    assert "layer_idx" not in fn.func.__code__.co_varnames
+
+
+def test_product_path_has_no_cpu_fallback():
+    from pbs_attn_amd import permuted_block_sparse_attn_fwd
+    from pbs_attn_amd._lib import PbsHipError
+    q = torch.zeros((1, 2, 512, 128), dtype=torch.bfloat16)
+    with pytest.raises(PbsHipError):
+        permuted_block_sparse_attn_fwd(q, q, q, 128, 256, 0.9, True)
+
+
+# ------------------------------------------------------------------ patcher on tiny models
+def _tiny(kind, layers=2):
+    from transformers import LlamaConfig, LlamaForCausalLM, Qwen2Config, Qwen2ForCausalLM
+    torch.manual_seed(0)
+    common = dict(hidden_size=64, intermediate_size=128, num_hidden_layers=layers, num_attention_heads=4,
+                  num_key_value_heads=2, vocab_size=97, max_position_embeddings=512)
+    if kind == "llama":
+        return LlamaForCausalLM(LlamaConfig(head_dim=16, **common)).eval()
+    return Qwen2ForCausalLM(Qwen2Config(**common)).eval()
+
+
+def _oracle_prefill(**kw):
+    def oracle_prefill(query_states, key_states, value_states):
+        return O.permuted_block_sparse_attn_fwd(query_states, key_states, value_states, **kw)
+    return oracle_prefill
+
+
+@pytest.mark.parametrize("kind", ["llama", "qwen2"])
+def test_patched_model_with_full_selection_equals_unpatched(kind):
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill
+    model = _tiny(kind)
+    ids = torch.randint(0, 97, (2, 48), generator=torch.Generator().manual_seed(1))
+    with torch.no_grad():
+        ref = model(ids).logits
+        apply_patch_with_prefill(model, _oracle_prefill(block_size=8, segment_size=16, threshold=1))
+        got = model(ids).logits
+    assert torch.allclose(got, ref, atol=2e-4)
+    for layer in model.model.layers:
+        assert hasattr(layer.self_attn, "original_forward")
+
+
+def test_skip_layers_and_errors():
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill
+    model = _tiny("llama", layers=3)
+    apply_patch_with_prefill(model, _oracle_prefill(block_size=8, segment_size=16, threshold=1), skip_layers=[1])
+    assert hasattr(model.model.layers[0].self_attn, "original_forward")
+    assert not hasattr(model.model.layers[1].self_attn, "original_forward")
+    with pytest.raises(ValueError):
+        apply_patch_with_prefill(torch.nn.Linear(2, 2), _oracle_prefill(block_size=8, segment_size=16, threshold=1))
+    m2 = _tiny("llama")
+    apply_patch_with_prefill(m2, None)
+    with pytest.raises(RuntimeError, match="prefill_fn required"):
+        m2(torch.randint(0, 97, (1, 8)))
+
+
+def test_generate_prefill_then_decode_uses_unpermuted_cache():
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill
+    model = _tiny("llama")
+    ids = torch.randint(0, 97, (1, 40), generator=torch.Generator().manual_seed(2))
+    with torch.no_grad():
+        ref = model.generate(ids, max_new_tokens=4, do_sample=False)
+        apply_patch_with_prefill(model, _oracle_prefill(block_size=8, segment_size=16, threshold=1))
+        got = model.generate(ids, max_new_tokens=4, do_sample=False)
+    assert torch.equal(got, ref)
+
+
+def test_layer_idx_is_passed_when_the_kernel_asks_for_it():
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill
+    seen = []
+
+    def prefill_with_layer(query_states, key_states, value_states, layer_idx=None):
+        seen.append((layer_idx, key_states.shape[1]))
+        return torch.nn.functional.scaled_dot_product_attention(query_states, key_states, value_states, is_causal=True)
+
+    model = _tiny("qwen2")
+    apply_patch_with_prefill(model, partial(prefill_with_layer))
+    with torch.no_grad():
+        model(torch.randint(0, 97, (1, 12)))
+    assert seen == [(0, 4), (1, 4)]            # K/V repeated to the 4 query heads
+
+
+def test_native_gqa_kernels_get_unrepeated_kv():
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill
+    shapes = []
+
+    def gqa_prefill(query_states, key_states, value_states):
+        shapes.append(key_states.shape[1])
+        return O.permuted_block_sparse_attn_fwd(query_states, key_states, value_states, 8, 16, 1)
+    gqa_prefill.native_gqa = True
+    model = _tiny("llama")
+    ids = torch.randint(0, 97, (1, 40), generator=torch.Generator().manual_seed(3))
+    with torch.no_grad():
+        ref = model(ids).logits
+        apply_patch_with_prefill(model, gqa_prefill)
+        got = model(ids).logits
+    assert shapes == [2, 2] and torch.allclose(got, ref, atol=2e-4)
+
+
+def test_synthetic_generators_are_seeded_and_shaped():
+    from pbs_attn_amd.synth import WORKLOADS, make_qkv
+    a = make_qkv(1, 4, 2, 256, 128, "uniform_heavy", seed=5)
+    b = make_qkv(1, 4, 2, 256, 128, "uniform_heavy", seed=5)
+    assert all(torch.equal(x, y) for x, y in zip(a, b))
+    assert a[0].shape == (1, 4, 256, 128) and a[1].shape == (1, 2, 256, 128) and a[0].dtype == torch.bfloat16
+    for kind in ("span_heavy", "local_window", "strong_heavy"):
+        q, k, v = make_qkv(2, 4, 1, 640, 128, kind, seed=1)
+        assert q.shape == (2, 4, 640, 128) and torch.isfinite(q.float()).all()
+    assert set(WORKLOADS) >= {"cfg0", "cfg1", "cfg2", "cfg3"}
