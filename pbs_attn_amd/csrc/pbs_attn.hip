@@ -1,28 +1,45 @@
 // Block-sparse flash-attention forward over permuted keys (bf16, head_dim 128).
 //
-// One workgroup = one 128-query block of one head; its four waves own 32 queries
-// each and walk the row's list of selected key blocks.  Per key block the K tile
-// (128 keys x 128 d, row-major) and the V tile (stored transposed, 128 d x 128
-// keys) are copied asynchronously straight into LDS (no registers) with a 16-byte
-// XOR swizzle -- the next K tile while softmax and P.V run, the next V tile while
-// the next S is computed -- and consumed by
-// v_mfma_f32_32x32x16_bf16 in the transposed formulation
-//     S^T = K Q^T            (rows = keys,  columns = queries)
-//     O^T += V^T P^T         (rows = d,     columns = queries)
-// so that every lane owns ONE query column: row max / row sum are in-lane
-// reductions plus one exchange with lane^32, and the S^T accumulator registers
-// are, after conversion to bf16, exactly the B operand of the second product
-// (the key rows of each 32-row MFMA tile are fed in the order that makes this so).
-// Softmax runs in the exp2 domain in fp32; P is rounded to bf16 before P.V and
-// the row sum uses the unrounded values; the output is normalised at the end.
-// Key blocks of the query block's own segment take the element mask
-// "original key position > query position"; earlier segments need no mask.
+// Work decomposition
+//   One workgroup (8 waves, two per SIMD) owns TWO adjacent 128-query blocks of one head.  Waves
+//   0-3 serve the first block, waves 4-7 the second, 32 queries per wave.  The two visit lists
+//   (ascending key-block indices) are merged once into LDS; every merged key block is copied ONCE
+//   into LDS for both query blocks, which halves the L2 -> LDS traffic and doubles the time a tile
+//   stays in flight.  K and V tiles are double-buffered (2 x 64 KB) and fetched one tile ahead with
+//   asynchronous global -> LDS copies (no registers), one workgroup barrier per tile.
+// Data layout
+//   K tile: 128 keys x 128 d row-major; V tile: stored TRANSPOSED in HBM by the gather kernel,
+//   128 d x 128 keys.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
+//   (row & 15): v_mfma fragment reads (row = lane % 32, 16 bytes) are bank-conflict free.
+// Math (transposed formulation, v_mfma_f32_32x32x16_bf16)
+//     S^T = K Q^T   (rows = keys, columns = queries)      O^T += V^T P^T   (rows = d, columns = queries)
+//   Every lane owns ONE query column, so softmax statistics are per-lane values, and the S^T
+//   accumulator registers are, after conversion to bf16, exactly the B operand of the second
+//   product (the key rows of each 32-row MFMA tile are fed in the order that makes this so).
+//   Softmax runs in the exp2 domain in fp32; P is rounded to bf16 before P.V and the row sum uses
+//   the unrounded values; the output is normalised once at the end.
+// Tile kinds
+//   * fast tiles (earlier segments, after the first): a software pipeline over the four 32-key
+//     sub-tiles -- S of sub-tile k+1, exponentials of sub-tile k and P.V of sub-tile k-1 are issued
+//     interleaved, LDS fragments are read three slots ahead.  Exponentials are taken against a LAZY
+//     reference maximum: it is not updated per tile; a row sum of one tile above 2^14 triggers a
+//     uniform rescale (exact, all terms share the reference); an overflow marks the row and the
+//     whole workgroup redoes it without speculation.
+//   * careful tiles (the first tile of a row, tiles of the query block's own segment, and the redo
+//     pass): all of S first, exact running maximum, element mask "original key position > query
+//     position" in the own segment.
 #include "pbs_common.h"
 
 namespace {
 
 constexpr int D = 128;
 constexpr int BS = 128;
+constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
+constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
+constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096)
+constexpr uint32_t LDS_MISC = LDS_LIST + 8192;    // ints: [0] merged count, [1] redo flag, [16..528) scan
+constexpr uint32_t LDS_TOTAL = LDS_MISC + 4096;   // 143 360 bytes of the CU's 160 KB
+constexpr int PREFETCH_SLOTS = 3;                 // LDS fragment reads run this many slots ahead
 
 struct AttnArgs {
   const uint16_t* q;
@@ -37,68 +54,110 @@ struct AttnArgs {
   float scale_log2;
 };
 
-// row of the 32-row MFMA tile -> key of the 32-key sub-tile, chosen so that the
-// accumulator registers 8u..8u+7 of lane-half g hold keys 16u + 8g + 0..7
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+// row of the 32-row MFMA tile -> key of the 32-key sub-tile, chosen so that the accumulator
+// registers 8u..8u+7 of lane-half g hold keys 16u + 8g + 0..7
 __device__ __forceinline__ int mfma_row_to_key(int i) {
   const int a = i >> 3, g = (i >> 2) & 1, c = i & 3;
   return 16 * (a >> 1) + 8 * g + 4 * (a & 1) + c;
 }
 
-// ---- asynchronous global -> LDS copy of one 32 KB tile ------------------------------------
-// LDS keeps a tile as 128 rows x 16 chunks of 16 bytes; physical chunk p of row r holds logical
-// chunk p ^ (r & 15) (bank-conflict-free fragment reads).  global_load_lds_dwordx4 writes lane l
-// at M0 + 16 l, so one wave instruction fills 4 consecutive rows and the swizzle is applied on
-// the GLOBAL side: lane l of wave w fetches chunk (l & 15) ^ (row & 15) of row 4 w + 16 n + (l >> 4).
-// That chunk does not depend on n: one per-lane byte offset serves the eight loads of a tile,
-// the tile base and the LDS base advance by 4096 bytes per load in scalar registers.
-// The copy is issued from inline assembly so that the compiler does not order later LDS reads
-// of OTHER buffers behind it; completion is awaited with explicit s_waitcnt vmcnt(N).
+// ---- asynchronous global -> LDS copy of one 32 KB tile by 512 threads ----------------------
+// global_load_lds_dwordx4 writes lane l at M0 + 16 l, so one wave instruction fills 4 consecutive
+// LDS rows and the chunk swizzle is applied on the GLOBAL side: lane l of wave w fetches chunk
+// (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4).  That chunk does not depend on n: one
+// per-lane byte offset serves the four loads, tile base and LDS base advance by 8192 bytes in
+// scalar registers.  The copy is issued from inline assembly so that the compiler does not order
+// later LDS reads of the OTHER buffer behind it; completion is awaited with s_waitcnt vmcnt(0)
+// before the barrier that publishes the tile.
 __device__ __forceinline__ uint32_t async_lane_offset(int wave, int lane) {
   const int row = 4 * wave + (lane >> 4);
   const int c = (lane & 15) ^ (row & 15);
   return (uint32_t)((row * D + c * 8) * 2);
 }
 
-__device__ __forceinline__ void stage_tile_async(const uint16_t* src, const uint16_t* lds, int wave, uint32_t lane_off) {
-  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane(
-      (int)((uint32_t)(uintptr_t)(const __attribute__((address_space(3))) void*)lds + wave * 1024));
+__device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t lds_byte, int wave, uint32_t lane_off) {
+  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + wave * 1024));
   // readfirstlane returns int: widen through uint32_t or the low half would be sign-extended
   const uint64_t src0 = (uint64_t)(uintptr_t)src;
   const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
   const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
   const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
 #pragma unroll
-  for (int n = 0; n < 8; ++n) {
-    const uint64_t base = srcu + n * 4096;
-    const uint32_t m0v = lds0 + n * 4096;
+  for (int n = 0; n < 4; ++n) {
+    const uint64_t base = srcu + n * 8192;
+    const uint32_t m0v = lds0 + n * 8192;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(lane_off), "s"(base)
                  : "memory");
   }
 }
 
-#define PBS_WAIT_VMCNT_8() __builtin_amdgcn_s_waitcnt(0x0f78)   // at most the 8 newest loads outstanding
-#define PBS_WAIT_VMCNT_0() __builtin_amdgcn_s_waitcnt(0x0f70)
-
-__device__ __forceinline__ bf16x8 lds_frag(const uint16_t* lds, int row, int chunk) {
-  return *reinterpret_cast<const bf16x8*>(lds + row * D + ((chunk ^ (row & 15)) * 8));
+__device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const lds_u8*)(uintptr_t)byte_addr);
 }
 
-__global__ __launch_bounds__(256, 2) void sparse_attn_kernel(AttnArgs a) {
-  __shared__ __attribute__((aligned(16))) uint16_t lds_k[BS * D];
-  __shared__ __attribute__((aligned(16))) uint16_t lds_v[BS * D];
+#define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
 
-  // workgroup -> (head, query block): heads stay on one XCD (blockIdx % 8), long rows first
-  const int w_id = blockIdx.x;
-  const int xcd = w_id & 7, slot = w_id >> 3;
-  const int heads_per_xcd = (a.BH + 7) >> 3;
-  const int bh = (slot % heads_per_xcd) * 8 + xcd;
-  const int qb = a.nb - 1 - slot / heads_per_xcd;
-  if (bh >= a.BH) return;
-
+__global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // starts at LDS offset 0
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j = lane & 31, gh = lane >> 5;
+  const int grp = wave >> 2, wq = wave & 3;
+
+  // workgroup -> (head, pair of query blocks): heads stay on one XCD (blockIdx % 8), long rows first
+  const int npair = (a.nb + 1) >> 1;
+  const int w_id = blockIdx.x;
+  const int xcd = w_id & 7, slot_id = w_id >> 3;
+  const int heads_per_xcd = (a.BH + 7) >> 3;
+  const int bh = (slot_id % heads_per_xcd) * 8 + xcd;
+  const int pair = npair - 1 - slot_id / heads_per_xcd;
+  if (bh >= a.BH) return;
   const int b = bh / a.Hq, h = bh % a.Hq;
-  const int qpos = qb * BS + 32 * wave + j;
+  const int qb = 2 * pair + grp;
+  const bool qb_valid = qb < a.nb;
+  const int qpos = qb * BS + 32 * wq + j;
+
+  uint16_t* mlist = reinterpret_cast<uint16_t*>(smem + LDS_LIST);
+  int* misc = reinterpret_cast<int*>(smem + LDS_MISC);
+
+  // ---- merged visit list of the two query blocks: entry = kb | use_first << 14 | use_second << 15
+  {
+    uint8_t* flags = smem;   // nb bytes; the tile area is free before the main loop
+    for (int i = tid; i < a.nb; i += 512) flags[i] = 0;
+    if (tid == 0) misc[1] = 0;
+    __syncthreads();
+    const int n0 = a.cnt[(int64_t)bh * a.nb + 2 * pair];
+    const int32_t* l0 = a.cols + ((int64_t)bh * a.nb + 2 * pair) * a.nb;
+    for (int i = tid; i < n0; i += 512) flags[l0[i]] = 1;
+    __syncthreads();
+    if (2 * pair + 1 < a.nb) {
+      const int n1 = a.cnt[(int64_t)bh * a.nb + 2 * pair + 1];
+      const int32_t* l1 = l0 + a.nb;
+      for (int i = tid; i < n1; i += 512) flags[l1[i]] |= 2;
+    }
+    __syncthreads();
+    const int per = (a.nb + 511) / 512;
+    const int k0 = tid * per, k1 = min(k0 + per, a.nb);
+    int c = 0;
+    for (int kb = k0; kb < k1; ++kb) c += flags[kb] ? 1 : 0;
+    int* scan = misc + 16;
+    scan[tid] = c;
+    __syncthreads();
+    for (int off = 1; off < 512; off <<= 1) {
+      const int v = tid >= off ? scan[tid - off] : 0;
+      __syncthreads();
+      scan[tid] += v;
+      __syncthreads();
+    }
+    int w = scan[tid] - c;
+    for (int kb = k0; kb < k1; ++kb)
+      if (flags[kb]) mlist[w++] = (uint16_t)(kb | (flags[kb] << 14));
+    if (tid == 511) misc[0] = scan[511];
+    __syncthreads();
+  }
+  const int n_tiles = misc[0];
+  const int own_first = (qb / a.bps) * a.bps;
 
   // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7
   bf16x8 qf[8];
@@ -110,146 +169,201 @@ __global__ __launch_bounds__(256, 2) void sparse_attn_kernel(AttnArgs a) {
       if (qpos >= a.S) qf[t] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
     }
   }
-
-  const int n_tiles = a.cnt[(int64_t)bh * a.nb + qb];
-  const int32_t* cols = a.cols + ((int64_t)bh * a.nb + qb) * a.nb;
-  const int own_first = (qb / a.bps) * a.bps;
   const uint16_t* pk = a.pk + (int64_t)bh * a.nb * BS * D;
   const uint16_t* pvt = a.pvt + (int64_t)bh * a.nb * BS * D;
   const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS;
 
-  f32x16 o[4];
+  // per-lane LDS byte offsets of the fragments inside buffer 0; XOR 0x8000 switches buffer.
+  //   K fragment (sub-tile ks, d-step t)      : koff[t] + ks * 8192
+  //   V fragment (keys 16 c .. 16 c + 15, dt) : voff[c] + dt * 8192
+  const int krow = mfma_row_to_key(j);
+  uint32_t koff[8], voff[8];
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt) o[dt] = (f32x16){0};
-  float m_run = -INFINITY, l_run = 0.f;
-
-  const int krow_in_tile = mfma_row_to_key(j);
+  for (int t = 0; t < 8; ++t) koff[t] = (uint32_t)(krow * 256 + (((2 * t + gh) ^ (krow & 15)) * 16));
+#pragma unroll
+  for (int c = 0; c < 8; ++c) voff[c] = LDS_V0 + (uint32_t)(j * 256 + (((2 * c + gh) ^ (j & 15)) * 16));
   const uint32_t lane_off = async_lane_offset(wave, lane);
+  const float c_log2 = a.scale_log2;
+  const uint32_t use_bit = 1u << (14 + grp);
 
-  // the visit list is read 64 entries at a time, one per lane, and handed out with readlane:
-  // no vector-memory wait sits between the asynchronous copies and their consumers
-  int col_cache = (lane < n_tiles) ? cols[lane] : 0;
-  int col_cache_next = 0;
-  if (n_tiles > 0) {
-    PBS_WAIT_VMCNT_0();
-    const int kb0 = __builtin_amdgcn_readlane(col_cache, 0);
-    stage_tile_async(pk + (int64_t)kb0 * BS * D, lds_k, wave, lane_off);
-    stage_tile_async(pvt + (int64_t)kb0 * BS * D, lds_v, wave, lane_off);
-  }
-
-  for (int it = 0; it < n_tiles; ++it) {
-    if ((it & 63) == 0) col_cache_next = (it + 64 + lane < n_tiles) ? cols[it + 64 + lane] : 0;
-    const int kb = __builtin_amdgcn_readlane(col_cache, it & 63);
-    const bool has_next = it + 1 < n_tiles;
-    if ((it & 63) == 63) col_cache = col_cache_next;
-    const int kb_next = has_next ? __builtin_amdgcn_readlane(col_cache, (it + 1) & 63) : 0;
-
-    PBS_WAIT_VMCNT_8();   // K(it) has landed; V(it) may still be in flight
-    __syncthreads();
-
-    // ---- S^T = K Q^T
-    f32x16 s[4];
+  for (int attempt = 0; attempt < 2; ++attempt) {
+    const bool careful_only = attempt == 1;
+    f32x16 o[4];
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      s[ks] = (f32x16){0};
-      const int row = 32 * ks + krow_in_tile;
-#pragma unroll
-      for (int t = 0; t < 8; ++t) s[ks] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(lds_k, row, 2 * t + gh), qf[t], s[ks], 0, 0, 0);
+    for (int dt = 0; dt < 4; ++dt) o[dt] = (f32x16){0};
+    float m_ref = -INFINITY;   // reference maximum, identical in lanes j and j + 32
+    float l_part = 0.f;        // row sum of this lane's half of the keys
+    bool first = true, poisoned = false;
+
+    __syncthreads();   // list build / previous attempt are done with the tile buffers
+    if (n_tiles > 0) {
+      const int kb0 = mlist[0] & 0x3fff;
+      stage_tile_async(pk + (int64_t)kb0 * BS * D, 0, wave, lane_off);
+      stage_tile_async(pvt + (int64_t)kb0 * BS * D, LDS_V0, wave, lane_off);
     }
-    __syncthreads();      // every wave is done with K(it): the next K tile may overwrite it
-    if (has_next) stage_tile_async(pk + (int64_t)kb_next * BS * D, lds_k, wave, lane_off);
+    for (int it = 0; it < n_tiles; ++it) {
+      const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it]);
+      const int kb = ent & 0x3fff;
+      const bool has_next = it + 1 < n_tiles;
+      const int kb_next = has_next ? (__builtin_amdgcn_readfirstlane((int)mlist[it + 1]) & 0x3fff) : 0;
+      const uint32_t bufx = (it & 1) ? 0x8000u : 0u;
+      __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` has landed
+      __syncthreads();                      // every share has; every wave is done with tile it - 1
+      if (has_next) {
+        stage_tile_async(pk + (int64_t)kb_next * BS * D, bufx ^ 0x8000u, wave, lane_off);
+        stage_tile_async(pvt + (int64_t)kb_next * BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+      }
+      if (!(ent & use_bit) || !qb_valid) continue;
+      const bool masked = kb >= own_first;
 
-    // ---- element mask inside the query block's own segment
-    if (kb >= own_first) {
+      if (first || masked || careful_only) {
+        // ---------------- careful tile
+        first = false;
+        f32x16 s[4];
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        __builtin_amdgcn_sched_barrier(0);   // keep the index loads of one sub-tile at a time in flight
+        for (int ks = 0; ks < 4; ++ks) {
+          s[ks] = (f32x16){0};
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          const int p = kb * BS + 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1);
-          const int4 ki = *reinterpret_cast<const int4*>(idx + p);
-          if (ki.x > qpos) s[ks][4 * a4 + 0] = -INFINITY;
-          if (ki.y > qpos) s[ks][4 * a4 + 1] = -INFINITY;
-          if (ki.z > qpos) s[ks][4 * a4 + 2] = -INFINITY;
-          if (ki.w > qpos) s[ks][4 * a4 + 3] = -INFINITY;
+          for (int t = 0; t < 8; ++t) s[ks] = PBS_MFMA(ldsf((koff[t] ^ bufx) + ks * 8192), qf[t], s[ks]);
+        }
+        if (masked) {
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+            __builtin_amdgcn_sched_barrier(0);   // keep the index loads of one sub-tile at a time in flight
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+              const int p = kb * BS + 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1);
+              const int4 ki = *reinterpret_cast<const int4*>(idx + p);
+              if (ki.x > qpos) s[ks][4 * a4 + 0] = -INFINITY;
+              if (ki.y > qpos) s[ks][4 * a4 + 1] = -INFINITY;
+              if (ki.z > qpos) s[ks][4 * a4 + 2] = -INFINITY;
+              if (ki.w > qpos) s[ks][4 * a4 + 3] = -INFINITY;
+            }
+          }
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[ks][r]);
+        mx = fmaxf(mx, xhalf_f32(mx));
+        const float m_new = fmaxf(m_ref, mx * c_log2);
+        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
+        float rs = 0.f;
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const float p = __builtin_amdgcn_exp2f(s[ks][r] * c_log2 - m_use);
+            s[ks][r] = p;
+            rs += p;
+          }
+        l_part = l_part * alpha + rs;
+        m_ref = m_new;
+        if (__any(alpha != 1.0f)) {
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+          for (int u = 0; u < 2; ++u) {
+            bf16x8 pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s[ks][8 * u + e];
+#pragma unroll
+            for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff[2 * ks + u] ^ bufx) + dt * 8192), pf, o[dt]);
+          }
+      } else {
+        // ---------------- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved,
+        //   S of sub-tile s (s <= 3), exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2);
+        //   S and P are double-buffered by sub-tile parity.  One scheduling barrier per slot keeps the order.
+        const float negm = -m_ref;
+        float rsum[4] = {0.f, 0.f, 0.f, 0.f};
+        f32x16 sbuf[2];
+        bf16x8 pbuf[2][2];
+        constexpr int R = PREFETCH_SLOTS + 1;
+        bf16x8 frk[R], frv[R];
+#pragma unroll
+        for (int n = 0; n < PREFETCH_SLOTS; ++n) frk[n % R] = ldsf((koff[n & 7] ^ bufx) + (n >> 3) * 8192);
+#pragma clang loop unroll(full)
+        for (int n = 0; n < 48; ++n) {
+          const int step = n >> 3, t = n & 7;
+          {   // fragment reads for slot n + PREFETCH_SLOTS
+            const int m = n + PREFETCH_SLOTS, mstep = m >> 3, mt = m & 7;
+            if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff[mt] ^ bufx) + mstep * 8192);
+            if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff[2 * (mstep - 2) + (mt >> 2)] ^ bufx) + (mt & 3) * 8192);
+          }
+          if (step <= 3) {
+            const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
+            sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
+          }
+          if (step >= 2) o[t & 3] = PBS_MFMA(frv[n % R], pbuf[step & 1][t >> 2], o[t & 3]);
+          if (step >= 1 && step <= 4) {
+            const int sb = (step - 1) & 1, r = 2 * t;
+            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sbuf[sb][r], c_log2, negm));
+            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sbuf[sb][r + 1], c_log2, negm));
+            rsum[t & 3] += e0;
+            rsum[(t + 2) & 3] += e1;
+            pbuf[sb][r >> 3][r & 7] = (__bf16)e0;
+            pbuf[sb][r >> 3][(r & 7) + 1] = (__bf16)e1;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        const float rs = (rsum[0] + rsum[1]) + (rsum[2] + rsum[3]);
+        l_part += rs;
+        // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
+        // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
+        if (__any(rs > 16384.0f)) {
+          const float big = fmaxf(rs, xhalf_f32(rs));
+          if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
+          const float m_new = (big > 16384.0f) ? m_ref + __builtin_amdgcn_logf(big) : m_ref;
+          const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+          m_ref = m_new;
+          l_part *= alpha;
+#pragma unroll
+          for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
         }
       }
     }
-
-    // ---- online softmax (exp2 domain), one query per lane pair (lane, lane^32)
-    float mx = -INFINITY;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[ks][r]);
-    mx = fmaxf(mx, xhalf_f32(mx));
-    const float m_new = fmaxf(m_run, mx * a.scale_log2);
-    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_use);
-    float rs = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float p = __builtin_amdgcn_exp2f(s[ks][r] * a.scale_log2 - m_use);
-        s[ks][r] = p;
-        rs += p;
-      }
-    rs += xhalf_f32(rs);
-    l_run = l_run * alpha + rs;
-    m_run = m_new;
-    if (__any(alpha != 1.0f)) {   // the running maximum settles after a few tiles
-#pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-    }
-
-    if (has_next) PBS_WAIT_VMCNT_8();   // V(it) has landed (K(it+1) may be in flight)
-    else PBS_WAIT_VMCNT_0();
+    if (poisoned) misc[1] = 1;
     __syncthreads();
+    if (!careful_only && misc[1] != 0) continue;   // the whole workgroup redoes both rows without speculation
 
-    // ---- O^T += V^T P^T
+    // ---- epilogue: normalise, transpose through LDS (same swizzle), coalesced 16-byte stores
+    const float inv = 1.0f / (l_part + xhalf_f32(l_part));
+    uint16_t* os = reinterpret_cast<uint16_t*>(smem) + grp * (BS * D);
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks)
+    for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int u = 0; u < 2; ++u) {
-        bf16x8 pf;
+      for (int a4 = 0; a4 < 4; ++a4) {
+        const int row = 32 * wq + j;
+        const int c = 4 * dt + a4;   // 16-byte chunk of d = 32 dt + 8 a4 + 4 gh + 0..3
+        bf16x4 v4;
 #pragma unroll
-        for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s[ks][8 * u + e];
-#pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
-          o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(lds_frag(lds_v, 32 * dt + j, 4 * ks + 2 * u + gh), pf, o[dt], 0, 0, 0);
+        for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][4 * a4 + cc] * inv);
+        *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * gh) = v4;
       }
-    __syncthreads();      // every wave is done with V(it)
-    if (has_next) stage_tile_async(pvt + (int64_t)kb_next * BS * D, lds_v, wave, lane_off);
-  }
-
-  // ---- epilogue: normalise, transpose through LDS (same swizzle), coalesced 16-byte stores
-  __syncthreads();
-  const float inv = 1.0f / l_run;
-  uint16_t* os = lds_k;
+    __syncthreads();
+    if (qb_valid) {
+      uint16_t* obase = a.o + b * a.o_sb + h * a.o_sh;
+      const int t256 = tid & 255;
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-    for (int a4 = 0; a4 < 4; ++a4) {
-      const int row = 32 * wave + j;
-      const int c = 4 * dt + a4;   // 16-byte chunk of d = 32 dt + 8 a4 + 4 gh + 0..3
-      bf16x4 v4;
-#pragma unroll
-      for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][4 * a4 + cc] * inv);
-      *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * gh) = v4;
+      for (int n = 0; n < 8; ++n) {
+        const int ci = t256 + 256 * n;
+        const int row = ci >> 4, c = ci & 15;
+        const int pos = qb * BS + row;
+        if (pos < a.S)
+          *reinterpret_cast<u32x4*>(obase + (int64_t)pos * a.o_ss + c * 8) =
+              *reinterpret_cast<const u32x4*>(os + row * D + ((c ^ (row & 15)) * 8));
+      }
     }
-  __syncthreads();
-  uint16_t* obase = a.o + b * a.o_sb + h * a.o_sh;
-#pragma unroll
-  for (int n = 0; n < 8; ++n) {
-    const int ci = tid + 256 * n;
-    const int row = ci >> 4, c = ci & 15;
-    const int pos = qb * BS + row;
-    if (pos < a.S)
-      *reinterpret_cast<u32x4*>(obase + (int64_t)pos * a.o_ss + c * 8) =
-          *reinterpret_cast<const u32x4*>(os + row * D + ((c ^ (row & 15)) * 8));
+    break;
   }
 }
 
@@ -274,9 +388,15 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
   a.BH = B * Hq; a.Hq = Hq; a.S = S; a.nb = (S + BS - 1) / BS; a.bps = segment_size / block_size;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
   a.scale_log2 = softmax_scale * 1.4426950408889634f;
+  PBS_REQUIRE(a.nb <= 4096, "pbs_sparse_attn_fwd: more than 4096 blocks per sequence (%d)", a.nb);
   const int heads_per_xcd = (a.BH + 7) / 8;
-  const int64_t n_wg = (int64_t)8 * heads_per_xcd * a.nb;
+  const int64_t n_wg = (int64_t)8 * heads_per_xcd * ((a.nb + 1) / 2);
   PBS_REQUIRE(n_wg < (1ll << 31), "pbs_sparse_attn_fwd: launch too large");
-  hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(256), 0, (hipStream_t)stream, a);
+  hipError_t attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
+  if (attr != hipSuccess) {
+    pbs_set_error("pbs_sparse_attn_fwd: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
+    return (int)attr;
+  }
+  hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(512), LDS_TOTAL, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_sparse_attn_fwd");
 }
