@@ -2,6 +2,7 @@
 // over all keys of the complete segments (no causal mask).
 //
 // Three launches, K is read twice and never re-materialised:
+//   (all exponentials are base 2 on logits pre-multiplied by log2(e))
 //   1. score_partial : per (head, key chunk) online (max, sum-exp) of every query row
 //   2. score_reduce  : fold the chunk partials into (row max, 1 / row sum)
 //   3. score_final   : recompute the logits and emit the per-key mean probability
@@ -22,7 +23,7 @@ struct ScoreArgs {
   int B, Hq, Hkv, S, Sc;
   int64_t q_sb, q_sh, q_ss;
   int64_t k_sb, k_sh, k_ss;
-  float sqrt_d;
+  float inv_sqrt_d;
   float* part;    // (B*Hq, nchunk, NQ, 2)
   float* stats;   // (B*Hq, NQ, 2)  (max, 1/sum)
   float* scores;  // (B*Hq, Sc)
@@ -34,8 +35,15 @@ __device__ __forceinline__ bf16x8 load_frag(const uint16_t* row_ptr, int t, int 
   return *reinterpret_cast<const bf16x8*>(row_ptr + 16 * t + 8 * half);
 }
 
-__device__ __forceinline__ float logit_round(float acc, float sqrt_d) {
-  return round_bf16(round_bf16(acc) / sqrt_d);
+// fp32 accumulator -> the bf16 logit a bf16 matmul followed by a bf16 divide by sqrt(D) yields, times
+// log2(e): round to bf16, scale (multiplication by the reciprocal; it differs from the true quotient by
+// at most one fp32 ulp, which survives the second bf16 rounding only for values within 2^-16 of a tie),
+// round to bf16.  Hardware conversions (round to nearest even).
+__device__ __forceinline__ float hw_round_bf16(float x) {
+  return bf16_bits_to_f32((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x));
+}
+__device__ __forceinline__ float logit_log2(float acc, float inv_sqrt_d) {
+  return hw_round_bf16(hw_round_bf16(acc) * inv_sqrt_d) * 1.4426950408889634f;
 }
 
 // One wave per query head of the KV group; the four waves of a workgroup walk
@@ -100,14 +108,14 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
             float v[16], mx = -INFINITY;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              v[r] = logit_round(acc[r], a.sqrt_d);
+              v[r] = logit_log2(acc[r], a.inv_sqrt_d);
               mx = fmaxf(mx, v[r]);
             }
             const float m_new = fmaxf(m_run[qt], mx);
             float sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sum += __expf(v[r] - m_new);
-            l_run[qt] = l_run[qt] * __expf(m_run[qt] - m_new) + sum;
+            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(v[r] - m_new);
+            l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + sum;
             m_run[qt] = m_new;
           }
         } else {
@@ -122,7 +130,7 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
             for (int r = 0; r < 16; ++r) {
               const int qrow = 32 * qt + 8 * (r >> 2) + 4 * half + (r & 3);
               const float mx = s_stats[wave][qrow][0], inv = s_stats[wave][qrow][1];
-              accp += __expf(logit_round(acc[r], a.sqrt_d) - mx) * inv;
+              accp += __builtin_amdgcn_exp2f(logit_log2(acc[r], a.inv_sqrt_d) - mx) * inv;
             }
           }
           accp += xhalf_f32(accp);
@@ -134,7 +142,7 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
         for (int qt = 0; qt < 4; ++qt) {
           const float m_o = xhalf_f32(m_run[qt]), l_o = xhalf_f32(l_run[qt]);
           const float m_new = fmaxf(m_run[qt], m_o);
-          const float l_new = l_run[qt] * __expf(m_run[qt] - m_new) + l_o * __expf(m_o - m_new);
+          const float l_new = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + l_o * __builtin_amdgcn_exp2f(m_o - m_new);
           if (half == 0) {
             float* p = a.part + (((int64_t)bh * a.nchunk + chunk) * NQ + 32 * qt + j) * 2;
             p[0] = m_new;
@@ -153,7 +161,7 @@ __global__ __launch_bounds__(NQ) void score_reduce_kernel(ScoreArgs a) {
   for (int c = 0; c < a.nchunk; ++c) {
     const float mc = p[((int64_t)c * NQ + qrow) * 2], lc = p[((int64_t)c * NQ + qrow) * 2 + 1];
     const float m_new = fmaxf(m, mc);
-    l = l * __expf(m - m_new) + lc * __expf(mc - m_new);
+    l = l * __builtin_amdgcn_exp2f(m - m_new) + lc * __builtin_amdgcn_exp2f(mc - m_new);
     m = m_new;
   }
   a.stats[((int64_t)bh * NQ + qrow) * 2] = m;
@@ -195,7 +203,7 @@ extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.Sc = Sc;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
-  a.sqrt_d = (float)sqrt((double)head_dim);
+  a.inv_sqrt_d = (float)(1.0 / sqrt((double)head_dim));
   a.chunk_keys = chunk_keys_for(Hq / Hkv);
   a.nchunk = chunks_for(Sc, a.chunk_keys);
   a.part = (float*)workspace;

@@ -73,17 +73,34 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
     }
     bitonic_sort_lds(keys, a.n_pow2);
     if (threadIdx.x == 0) {
+      // sequential float64 running sum, every prefix rounded to float32 (what torch's CPU cumsum does).
+      // Chunks of 16 sorted values are fetched together and summed without branches, so the serial
+      // chain is 16 double additions; the first qualifying rank is picked from bit masks afterwards.
       const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
       double c = 0.0;
       int first = -1;
-      for (int r = 0; r < nb; ++r) {
-        const float v = desc_key_value(keys[r]);
-        c += (double)v;
-        if ((float)c >= thr) {
-          first = r;
+      for (int r0 = 0; r0 < nb; r0 += 16) {
+        float v[16];
+#pragma unroll
+        for (int u = 0; u < 16; ++u) v[u] = desc_key_value(keys[min(r0 + u, a.n_pow2 - 1)]);
+        uint32_t reach = 0, zero = 0;
+#pragma unroll
+        for (int u = 0; u < 16; ++u) {
+          c += (double)v[u];
+          reach |= ((float)c >= thr ? 1u : 0u) << u;
+          zero |= (v[u] == 0.f ? 1u : 0u) << u;
+        }
+        const uint32_t valid = (nb - r0 >= 16) ? 0xffffu : ((1u << (nb - r0)) - 1u);
+        reach &= valid;
+        zero &= valid;
+        // a zero ends the search (sorted: nothing positive follows) unless the threshold is reached
+        // at or before it
+        const int ur = reach ? __builtin_ctz(reach) : 32, uz = zero ? __builtin_ctz(zero) : 32;
+        if (ur <= uz && ur < 32) {
+          first = r0 + ur;
           break;
         }
-        if (v == 0.f) break;  // sorted: nothing positive follows, the sum cannot grow
+        if (uz < 32) break;
       }
       s_first = first;
     }
@@ -96,11 +113,16 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
     const int fb = a.first_blk[row];
     if (fb >= 0 && fb < nb) flag[fb] = 1;
   }
-  // smallest original key position of each own-segment block
-  for (int o = seg_first; o < seg_end; ++o) {
-    if (threadIdx.x < a.bs) {
-      const int v = a.idx[(int64_t)row * nb * a.bs + (int64_t)o * a.bs + threadIdx.x];
-      atomicMin(&s_min[o - seg_first], v);
+  // smallest original key position of each own-segment block: one wave per block, shuffle reduction
+  {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int o = seg_first + wave; o < seg_end; o += (int)(blockDim.x >> 6)) {
+      const int32_t* src = a.idx + (int64_t)row * nb * a.bs + (int64_t)o * a.bs;
+      int v = INT_MAX;
+      for (int i = lane; i < a.bs; i += 64) v = min(v, src[i]);
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) v = min(v, __shfl_xor(v, off, 64));
+      if (lane == 0) s_min[o - seg_first] = v;
     }
   }
   __syncthreads();
