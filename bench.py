@@ -191,6 +191,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--traffic-calibration", action="store_true",
+                    help="also run one plain device copy of Q (known bytes) so that rocprofv3 --pmc FETCH_SIZE / "
+                         "WRITE_SIZE readings can be scaled")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -215,6 +218,12 @@ def main():
     res, inputs = run_workload(torch, args.workload, args.steps, args.warmup, overrides=overrides,
                                with_dense=not args.no_dense)
     log("[bench] " + json.dumps(res))
+    if args.traffic_calibration:
+        cfg, q = inputs[0], inputs[1]
+        dst = torch.empty_like(q)
+        dst.copy_(q)
+        torch.cuda.synchronize()
+        log(f"[bench] calibration copy: {q.numel() * q.element_size()} bytes read and written by one copy kernel")
 
     attn_s = res["stage_ms"]["sparse_attn"] * 1e-3
     achieved = res["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / attn_s / 1e12

@@ -1,0 +1,140 @@
+"""GPU checks at the benchmark's real sequence lengths, through size-independent
+properties (the CPU oracle cannot finish these sizes): known answers from a library
+routine, round trips, checksums, sortedness and the selection invariants."""
+import pytest
+import torch
+import torch.nn.functional as F
+
+from pbs_attn_amd import ops
+from pbs_attn_amd import pbs as P
+from pbs_attn_amd.synth import make_qkv
+from tests.util import assert_attn_close
+
+pytestmark = pytest.mark.gpu
+
+
+def _sdpa(q, k, v):
+    return F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+
+
+@pytest.mark.parametrize("S,Hq,Hkv,seg,kind", [(32768, 4, 1, 256, "uniform_heavy"), (32768, 4, 1, 1024, "uniform_heavy"),
+                                               (131072, 1, 1, 1024, "span_heavy"), (16384, 7, 1, 256, "local_window")])
+def test_full_selection_equals_dense_flash_attention(dev, S, Hq, Hkv, seg, kind):
+    # threshold = int 1 selects every causal block: the result must be plain causal attention
+    # whatever permutation the key sort produced
+    q, k, v = make_qkv(1, Hq, Hkv, S, 128, kind, seed=1, device=dev)
+    out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, seg, 1, True)
+    ref = _sdpa(q, k, v)
+    assert_attn_close(out, ref, what=f"threshold=1 vs SDPA at S={S}")
+
+
+def test_batched_gqa_7_to_1_against_dense_on_own_mask(dev):
+    # Qwen2.5-7B head grouping, batch 4: dense fp32 attention on the HIP path's own mask, sampled rows
+    B, Hq, Hkv, S, seg = 4, 28, 4, 4096, 256
+    q, k, v = make_qkv(B, Hq, Hkv, S, 128, "local_window", seed=2, device=dev)
+    perm = P.apply_permutation(q, k, v, 128, seg)
+    sel = P.permuted_block_selection(q, perm, 128, seg, 0.9)
+    out = ops.sparse_attn_fwd(q, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+    idx = perm.key_indices[:, :, :S].long()
+    pk, pv = perm.permuted_keys().float(), perm.permuted_values().float()
+    fm = sel["final_mask"]
+    pos = torch.arange(S, device=dev)
+    for qb in (0, 5, 17, 31):
+        rows = slice(qb * 128, qb * 128 + 128)
+        logits = q[:, :, rows].float() @ pk.transpose(-1, -2) / 128 ** 0.5
+        allowed = fm[:, :, qb][:, :, None, :].repeat_interleave(128, -1) & (idx[:, :, None, :] <= pos[rows].view(1, 1, -1, 1))
+        ref = torch.softmax(logits.masked_fill(~allowed, float("-inf")), -1) @ pv
+        assert_attn_close(out[:, :, rows], ref, what=f"q block {qb}")
+
+
+def test_permutation_gather_and_sort_properties_at_32k(dev):
+    S, seg, Hq, Hkv = 32768, 1024, 8, 2
+    q, k, v = make_qkv(1, Hq, Hkv, S, 128, "uniform_heavy", seed=3, device=dev)
+    scores = ops.score_keys(q, k, 128, seg)
+    assert torch.allclose(scores.sum(-1), torch.ones(1, Hq, device=dev), atol=2e-3)
+    perm = P.apply_permutation(q, k, v, 128, seg, scores=scores)
+    idx = perm.key_indices.long()
+    # a permutation of every segment's own range
+    srt = idx.view(1, Hq, -1, seg).sort(-1).values
+    assert torch.equal(srt, torch.arange(S, device=dev).view(1, 1, -1, seg).expand_as(srt))
+    # descending by score, ties by ascending index (the order torch's stable sort gives)
+    ref_idx = torch.sort(scores.view(1, Hq, -1, seg), dim=-1, descending=True, stable=True).indices
+    ref_idx = (ref_idx + torch.arange(0, S, seg, device=dev).view(1, 1, -1, 1)).view(1, Hq, S)
+    assert torch.equal(idx, ref_idx)
+    # gather round trip: scattering the permuted rows back restores K and V bit for bit
+    ke = k.repeat_interleave(Hq // Hkv, dim=1)
+    ve = v.repeat_interleave(Hq // Hkv, dim=1)
+    back = torch.empty_like(ke).scatter_(2, idx.unsqueeze(-1).expand(-1, -1, -1, 128), perm.permuted_keys())
+    assert torch.equal(back, ke)
+    back = torch.empty_like(ve).scatter_(2, idx.unsqueeze(-1).expand(-1, -1, -1, 128), perm.permuted_values())
+    assert torch.equal(back, ve)
+    # checksum of checksums: per-segment column sums are permutation invariant (exact in float64)
+    a = perm.permuted_keys().double().view(1, Hq, -1, seg, 128).sum(-2)
+    b = ke.double().view(1, Hq, -1, seg, 128).sum(-2)
+    assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("thr", [0.8, 0.9, 0.95])
+def test_selection_invariants_at_32k(dev, thr):
+    S, seg, Hq, Hkv = 32768, 256, 8, 2
+    nb, bps = S // 128, seg // 128
+    q, k, v = make_qkv(1, Hq, Hkv, S, 128, "uniform_heavy", seed=4, device=dev)
+    perm = P.apply_permutation(q, k, v, 128, seg)
+    sel = P.permuted_block_selection(q, perm, 128, seg, thr, force_select_first_block=False)
+    Pm, chosen, final = sel["block_attn_scores"], sel["block_mask"], sel["final_mask"]
+    qb = torch.arange(nb, device=dev)
+    cand = (qb.view(1, -1) // bps) < (qb.view(-1, 1) // bps)
+    own = (qb.view(1, -1) // bps) == (qb.view(-1, 1) // bps)
+    assert torch.isnan(Pm[:, :, :bps]).all() and not torch.isnan(Pm[:, :, bps:]).any()
+    Pz = torch.nan_to_num(Pm, nan=0.0).double()
+    assert (Pz[..., ~cand] == 0).all()
+    assert torch.allclose(Pz[:, :, bps:].sum(-1), torch.ones(1, Hq, nb - bps, device=dev, dtype=torch.double), atol=1e-4)
+    assert not (chosen & ~cand).any()                       # only candidates are ever selected
+    assert torch.equal(final, chosen | own)
+    mass = (Pz * chosen).sum(-1)[:, :, bps:]
+    assert (mass >= thr - 1e-5).all()                       # the threshold is reached ...
+    smallest = torch.where(chosen, Pz, torch.full_like(Pz, 2.0)).min(-1).values[:, :, bps:]
+    assert (mass - smallest < thr + 1e-5).all()             # ... and not without the smallest selected block
+    largest_out = torch.where(cand & ~chosen, Pz, torch.full_like(Pz, -1.0)).max(-1).values[:, :, bps:]
+    assert (largest_out <= smallest + 1e-12).all()          # a descending prefix
+    # the visit list is the final mask restricted to segments not after the query block's
+    cnt = sel["csr_cnt"]
+    visited = (final & ((qb.view(1, -1) // bps) <= (qb.view(-1, 1) // bps))).sum(-1)
+    assert ((cnt == visited) | (cnt == visited - 1)).all()  # one own-segment block may be provably all-masked
+    cols = sel["csr_cols"]
+    r = cols[0, 3, nb - 1, :cnt[0, 3, nb - 1]]
+    assert (r[1:] > r[:-1]).all() and final[0, 3, nb - 1, r.long()].all()
+
+
+def test_ones_value_and_linearity_at_32k(dev):
+    S, seg = 32768, 256
+    q, k, v = make_qkv(1, 4, 1, S, 128, "uniform_heavy", seed=5, device=dev)
+    fwd = lambda vv: P.permuted_block_sparse_attn_fwd(q, k, vv, 128, seg, 0.9, True)  # noqa: E731
+    ones = fwd(torch.ones_like(v))
+    assert torch.allclose(ones.float(), torch.ones_like(ones.float()), atol=8e-3)
+    # the output is linear in V for fixed Q, K (the mask does not depend on V)
+    a, b = fwd(v).float(), fwd((2 * v).to(v.dtype)).float()
+    assert torch.allclose(2 * a, b, atol=2e-2, rtol=2e-2)
+    # and repeatable bit for bit
+    assert torch.equal(fwd(v), fwd(v))
+
+
+@pytest.mark.parametrize("gain,what", [(3.0, "lazy rescale"), (12.0, "rescale by many octaves"), (60.0, "overflow -> redo without speculation")])
+def test_late_dominant_keys_take_the_rare_paths(dev, gain, what):
+    # keys far stronger than everything seen before them show up late in the visit list: the fast
+    # tiles' fixed reference maximum must be moved (exactly), or the row redone when exp2 overflowed
+    S, seg = 4096, 256
+    g = torch.Generator().manual_seed(7)
+    q = torch.randn((1, 2, S, 128), generator=g)
+    k = torch.randn((1, 2, S, 128), generator=g)
+    v = torch.randn((1, 2, S, 128), generator=g)
+    u = torch.zeros(128)
+    u[0] = 1.0
+    q = q + 4.0 * u
+    k[:, :, 2048:2048 + 128] += gain * 4.0 * u          # logit jump of about gain * 1.4 * 4 (and more for some queries)
+    k[:, :, 3000:3008] += 2 * gain * 4.0 * u
+    q, k, v = (t.to(torch.bfloat16).to(dev) for t in (q, k, v))
+    out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, seg, 1, True)
+    ref = _sdpa(q.float(), k.float(), v.float())
+    assert torch.isfinite(out.float()).all(), what
+    assert_attn_close(out, ref, what=what)
