@@ -182,6 +182,51 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     return res, (cfg, q, k, v)
 
 
+def density_without_permutation(torch, cfg, q, k, v):
+    """Block density of the same selection rule on UN-permuted keys (identity order through the same
+    kernels: strictly decreasing injected scores), the ablation that shows what the permutation buys."""
+    from pbs_attn_amd import pbs as P
+    B, Hq, S = cfg["B"], cfg["Hq"], cfg["S"]
+    bs, seg, thr = cfg["block"], cfg["segment"], cfg["threshold"]
+    sc = (S // seg) * seg
+    scores = -torch.arange(sc, device=q.device, dtype=torch.float32).view(1, 1, sc).expand(B, Hq, sc).contiguous()
+    perm = P.apply_permutation(q, k, v, bs, seg, scores=scores)
+    sel = P.permuted_block_selection(q, perm, bs, seg, thr, want_masks=False)
+    nb = (S + bs - 1) // bs
+    return int(sel["csr_cnt"].sum().item()) / (B * Hq * nb * (nb + 1) // 2)
+
+
+def run_report(torch, path, steps, warmup):
+    """Every BASELINE.json single-layer configuration + sweeps, written as a markdown table."""
+    runs = [("cfg0", {}), ("cfg1", {})]
+    runs += [("cfg1", {"segment": sg, "threshold": th}) for sg in (256, 1024) for th in (0.8, 0.9, 0.95)
+             if not (sg == 256 and th == 0.9)]
+    runs += [("cfg2", {}), ("cfg3", {}), ("cfg3", {"segment": 1024}),
+             ("cfg1", {"kind": "strong_heavy", "segment": 1024}), ("cfg2", {"kind": "strong_heavy"})]
+    lines = ["| workload | generator | S | B x Hq/Hkv | segment | thr | density | density w/o permutation | pass ms | "
+             "attn ms | attn TFLOP/s | % MFMA peak | dense SDPA ms | speed-up vs dense | score/sort/gather/estimate/select ms |",
+             "|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|"]
+    out = []
+    for name, ov in runs:
+        res, (cfg, q, k, v) = run_workload(torch, name, steps, warmup, overrides=ov, with_dense=True)
+        res["density_unpermuted"] = density_without_permutation(torch, cfg, q, k, v)
+        del q, k, v
+        torch.cuda.empty_cache()
+        st = res["stage_ms"]
+        lines.append(
+            f"| {name} | {res['generator']} | {res['S']} | {res['B']} x {res['Hq']}/{res['Hkv']} | {res['segment']} | "
+            f"{res['threshold']} | {res['density_vs_causal']:.3f} | {res['density_unpermuted']:.3f} | {res['ms_per_step']:.2f} | "
+            f"{st['sparse_attn']:.2f} | {res['effective_tflops_attn_kernel']:.0f} | "
+            f"{100 * res['effective_tflops_attn_kernel'] / PEAK_BF16_TFLOPS:.1f} | "
+            f"{res['dense_sdpa_ms']:.2f} | {res['dense_sdpa_ms'] / res['ms_per_step']:.2f} | "
+            f"{st.get('score', 0):.2f}/{st.get('sort', 0):.2f}/{st['gather']:.2f}/{st.get('estimate', 0):.2f}/{st['select']:.2f} |")
+        log(lines[-1])
+        out.append(res)
+    with open(path, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -194,6 +239,8 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--report", default=None, metavar="FILE.md",
+                    help="run every single-layer configuration and the sweeps, write a markdown table, and exit")
     ap.add_argument("--traffic-calibration", action="store_true",
                     help="also run one plain device copy of Q (known bytes) so that rocprofv3 --pmc FETCH_SIZE / "
                          "WRITE_SIZE readings can be scaled")
@@ -211,6 +258,10 @@ def main():
     from pbs_attn_amd import _lib
     _lib.load()
 
+    if args.report:
+        res = run_report(torch, args.report, args.steps, args.warmup)
+        print(json.dumps({"report": args.report, "rows": len(res)}), flush=True)
+        return
     overrides = {}
     if args.segment:
         overrides["segment"] = args.segment
