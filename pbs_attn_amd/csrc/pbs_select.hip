@@ -159,6 +159,202 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
   if (threadIdx.x == 255) a.csr_cnt[(int64_t)row * nb + qb] = s_scan[255];
 }
 
+
+// ---------------------------------------------------------------------------------------------
+// Wave-level variant (rows of up to 1024 blocks): ONE wave per row, the row lives in registers.
+//   * bitonic network on 64-bit composite keys, NPL keys per lane: strides below NPL are register
+//     compare-exchanges, larger strides exchange with lane ^ (stride / NPL); no barriers;
+//   * the running sum is first taken as a parallel float64 prefix (local prefixes + wave scan).  It
+//     differs from the sequential sum by < 1e-12, so "float32(prefix) >= threshold" is decided from it
+//     unless some prefix up to the first hit lies within 1e-11 of the float32 rounding boundary of the
+//     threshold; only then the exact sequential sum is evaluated (lane after lane).  Either way the
+//     decision is the one the sequential float64 sum gives;
+//   * flags, own-segment minima, masks and the compacted visit list as in the block-level kernel.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int lane_mask) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, lane_mask, 64), hi = __shfl_xor((uint32_t)(v >> 32), lane_mask, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ double shfl_up_f64(double v, int delta) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __shfl_up((uint32_t)u, delta, 64), hi = __shfl_up((uint32_t)(u >> 32), delta, 64);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)u, lane), hi = __builtin_amdgcn_readlane((int)(uint32_t)(u >> 32), lane);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
+template <int NPL>
+__device__ __forceinline__ void wave_bitonic_sort(uint64_t (&k)[NPL], int lane) {
+  constexpr int N = 64 * NPL;
+#pragma unroll
+  for (int size = 2; size <= N; size <<= 1) {
+#pragma unroll
+    for (int stride = size >> 1; stride > 0; stride >>= 1) {
+      if (stride >= NPL) {
+        const int lstride = stride / NPL;
+        const bool lower = (lane & lstride) == 0;
+        const bool up = (lane & (size / NPL)) == 0;
+        const bool keep_min = (lower == up);
+#pragma unroll
+        for (int r = 0; r < NPL; ++r) {
+          const uint64_t o = shfl_xor_u64(k[r], lstride);
+          const bool take = keep_min ? (o < k[r]) : (o > k[r]);
+          k[r] = take ? o : k[r];
+        }
+      } else {
+#pragma unroll
+        for (int r = 0; r < NPL; ++r) {
+          if ((r & stride) == 0) {
+            const int p = r | stride;
+            const bool up = (size >= NPL) ? ((lane & (size / NPL)) == 0) : ((r & size) == 0);
+            const uint64_t x = k[r], y = k[p];
+            const bool sw = (x > y) == up;
+            k[r] = sw ? y : x;
+            k[p] = sw ? x : y;
+          }
+        }
+      }
+    }
+  }
+}
+
+template <int NPL>
+__global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, int total_rows) {
+  extern __shared__ uint8_t smem_w[];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nb = a.nb;
+  const int nb_pad = (nb + 15) & ~15;
+  uint8_t* flag = smem_w + wave * nb_pad;
+  int* s_min = reinterpret_cast<int*>(smem_w + 4 * nb_pad) + wave * 256;
+  const int64_t rq = (int64_t)blockIdx.x * 4 + wave;   // (row, qb) flattened
+  if (rq >= total_rows) return;
+  const int row = (int)(rq / nb), qb = (int)(rq % nb);
+  const int seg_first = (qb / a.bps) * a.bps;
+  const int seg_end = min(seg_first + a.bps, nb);
+  const int64_t row_off = ((int64_t)row * nb + qb) * nb;
+
+  for (int kb = lane; kb < nb; kb += 64) flag[kb] = 0;
+
+  if (a.thr_is_int_one) {
+    for (int kb = lane; kb < seg_first; kb += 64) flag[kb] = 1;
+  } else {
+    const float* p = a.P + row_off;
+    uint64_t k[NPL];
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) {
+      const int i = lane * NPL + r;
+      uint64_t key = ~0ull;
+      if (i < nb) {
+        float v = p[i];
+        if (v != v) v = 0.f;
+        else if (v == INFINITY) v = FLT_MAX;
+        else if (v == -INFINITY) v = -FLT_MAX;
+        key = desc_stable_key(v, (uint32_t)i);
+      }
+      k[r] = key;
+    }
+    wave_bitonic_sort<NPL>(k, lane);
+
+    const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
+    float v[NPL];
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < nb) ? desc_key_value(k[r]) : 0.f;
+    // parallel float64 prefix
+    double loc[NPL];
+    double c = 0.0;
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) {
+      c += (double)v[r];
+      loc[r] = c;
+    }
+    double incl = c;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const double t = shfl_up_f64(incl, d);
+      if (lane >= d) incl += t;
+    }
+    double excl = shfl_up_f64(incl, 1);
+    if (lane == 0) excl = 0.0;
+    // float32 rounding boundary of the threshold (midpoint to its predecessor), as a double
+    const double mid = 0.5 * ((double)thr + (double)nextafterf(thr, -INFINITY));
+    uint32_t reach = 0, amb = 0;
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) {
+      const double cp = excl + loc[r];
+      reach |= ((float)cp >= thr ? 1u : 0u) << r;
+      amb |= (fabs(cp - mid) <= 1e-11 * fmax(1.0, fabs(mid)) ? 1u : 0u) << r;
+    }
+    int first = reach ? lane * NPL + __builtin_ctz(reach) : INT_MAX;
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) first = min(first, __shfl_xor(first, off, 64));
+    // ambiguous prefixes at or before the first hit?
+    bool my_amb = false;
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) my_amb |= ((amb >> r) & 1u) && (lane * NPL + r <= first) && (lane * NPL + r < nb);
+    if (__any(my_amb)) {
+      // exact sequential sum, lane after lane
+      double carry = 0.0;
+      first = INT_MAX;
+      for (int L = 0; L < 64; ++L) {
+        double cs = carry;
+        uint32_t rch = 0;
+#pragma unroll
+        for (int r = 0; r < NPL; ++r) {
+          cs += (double)v[r];
+          rch |= ((float)cs >= thr ? 1u : 0u) << r;
+        }
+        const uint32_t rl = (uint32_t)__builtin_amdgcn_readlane((int)rch, L);
+        carry = readlane_f64(cs, L);
+        if (rl) {
+          first = L * NPL + __builtin_ctz(rl);
+          break;
+        }
+      }
+    }
+    if (first >= nb) first = -1;   // never reached (padding ranks cannot qualify: they add zero)
+#pragma unroll
+    for (int r = 0; r < NPL; ++r)
+      if (lane * NPL + r <= first) flag[(uint32_t)k[r]] = 1;
+  }
+  __builtin_amdgcn_wave_barrier();
+  if (a.force_first && lane == 0) {
+    const int fb = a.first_blk[row];
+    if (fb >= 0 && fb < nb) flag[fb] = 1;
+  }
+  for (int o = seg_first; o < seg_end; ++o) {
+    const int32_t* src = a.idx + (int64_t)row * nb * a.bs + (int64_t)o * a.bs;
+    int mv = INT_MAX;
+    for (int i = lane; i < a.bs; i += 64) mv = min(mv, src[i]);
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) mv = min(mv, __shfl_xor(mv, off, 64));
+    if (lane == 0) s_min[o - seg_first] = mv;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+
+  const int q_last = min(qb * a.bs + a.bs - 1, a.S - 1);
+  int base = 0;
+  for (int kb0 = 0; kb0 < nb; kb0 += 64) {
+    const int kb = kb0 + lane;
+    bool visit = false;
+    if (kb < nb) {
+      const bool own = kb >= seg_first && kb < seg_end;
+      const uint8_t sf = flag[kb];
+      if (a.sel_mask) a.sel_mask[row_off + kb] = sf;
+      if (a.final_mask) a.final_mask[row_off + kb] = sf | (own ? 1 : 0);
+      visit = own ? (s_min[kb - seg_first] <= q_last) : (sf && kb < seg_first);
+    }
+    const uint64_t ballot = __ballot(visit);
+    if (visit && a.csr_cols) a.csr_cols[row_off + base + __popcll(ballot & ((1ull << lane) - 1ull))] = kb;
+    base += __popcll(ballot);
+  }
+  if (lane == 0) a.csr_cnt[(int64_t)row * nb + qb] = base;
+}
+
 }  // namespace
 
 extern "C" size_t pbs_select_blocks_workspace_bytes(int rows) { return (size_t)rows * sizeof(int32_t); }
@@ -187,6 +383,16 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   hipStream_t st = (hipStream_t)stream;
   if (force_select_first_block)
     hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size);
+  if (nb <= 1024) {
+    // one wave per row, four rows per workgroup
+    const int total = rows * nb;
+    const size_t lds_w = (size_t)4 * ((nb + 15) & ~15) + 4 * 256 * sizeof(int);
+    const dim3 grid((unsigned)((total + 3) / 4));
+    if (nb <= 64) hipLaunchKernelGGL(select_blocks_wave_kernel<1>, grid, dim3(256), lds_w, st, a, total);
+    else if (nb <= 256) hipLaunchKernelGGL(select_blocks_wave_kernel<4>, grid, dim3(256), lds_w, st, a, total);
+    else hipLaunchKernelGGL(select_blocks_wave_kernel<16>, grid, dim3(256), lds_w, st, a, total);
+    return pbs_check_launch("pbs_select_blocks");
+  }
   const size_t lds = (size_t)a.n_pow2 * sizeof(uint64_t) + (size_t)((nb + 15) / 16) * 16;
   hipLaunchKernelGGL(select_blocks_kernel, dim3(nb, rows), dim3(256), lds, st, a);
   return pbs_check_launch("pbs_select_blocks");

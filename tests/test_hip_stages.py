@@ -130,7 +130,7 @@ def _oracle_selection(P_scores, thr, idx_pad, nb, bps, force_first):
 
 @pytest.mark.parametrize("nb,bps,thr,force_first", [
     (8, 2, 0.9, True), (32, 2, 0.8, True), (32, 8, 0.95, False), (40, 8, 1.0, True), (40, 8, 1, True),
-    (33, 1, 0.5, True), (100, 4, 0.0, True), (64, 2, "tensor", True)])
+    (33, 1, 0.5, True), (100, 4, 0.0, True), (64, 2, "tensor", True), (300, 8, 0.9, True), (1030, 8, 0.9, True)])
 def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
     B, H, S = 2, 3, nb * 128 - 5
     g = torch.Generator().manual_seed(nb * 7 + bps)
@@ -154,9 +154,10 @@ def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
     cols, cnt = cols.cpu(), cnt.cpu()
     qseg = torch.arange(nb) // bps
     kmin = idx_pad.view(B, H, nb, 128).min(-1).values
+    qbs = range(nb) if nb <= 128 else list(range(0, nb, 37)) + [nb - 1]
     for b in range(B):
         for h in range(H):
-            for qb in range(nb):
+            for qb in qbs:
                 q_last = min(qb * 128 + 127, S - 1)
                 want = [kb for kb in range(nb) if ref_fin[b, h, qb, kb] and qseg[kb] <= qseg[qb]
                         and not (qseg[kb] == qseg[qb] and kmin[b, h, kb] > q_last)]
@@ -314,3 +315,20 @@ def test_error_behaviour(dev):
         P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 256, 0.9, True, query_pool_mode="median")
     with pytest.raises(AssertionError):
         P.permuted_block_sparse_attn_fwd(qd, kd[:, :, :256], vd[:, :, :256], 128, 256, 0.9, True)
+
+
+def test_select_blocks_prefix_on_the_float32_rounding_boundary(dev):
+    # a float64 prefix that lands exactly on the midpoint between float32(threshold) and its predecessor:
+    # the parallel prefix cannot decide, the kernel must fall back to the exact sequential sum
+    nb, bps = 64, 1
+    tiny = 2.0 ** -26
+    Pm = torch.zeros((1, 2, nb, nb))
+    Pm[0, 0, 40, 3] = 0.25
+    Pm[0, 0, 40, 7] = 0.25 - tiny           # 0.25 + (0.25 - 2^-26) = 0.5 - 2^-26 = the midpoint
+    Pm[0, 0, 40, 9] = 0.125
+    Pm[0, 1, 50, :10] = torch.tensor([0.3, 0.2 - tiny / 2, 1e-9, 1e-9, 0.1, 0.05, 0.05, 0.2, 0.01, 0.05])
+    idx_pad = torch.arange(nb * 128).expand(1, 2, -1).int()
+    for thr in (0.5, 0.5 - tiny, 0.7):
+        ref_sel, ref_fin = _oracle_selection(Pm, thr, idx_pad, nb, bps, False)
+        sel, fin, _, _ = ops.select_blocks(Pm.to(dev), thr, idx_pad.to(dev), nb * 128, 128, bps * 128, False)
+        assert torch.equal(sel.cpu(), ref_sel) and torch.equal(fin.cpu(), ref_fin), thr
