@@ -175,3 +175,24 @@ def test_synthetic_generators_are_seeded_and_shaped():
         q, k, v = make_qkv(2, 4, 1, 640, 128, kind, seed=1)
         assert q.shape == (2, 4, 640, 128) and torch.isfinite(q.float()).all()
     assert set(WORKLOADS) >= {"cfg0", "cfg1", "cfg2", "cfg3"}
+
+
+def test_bench_refuses_more_than_one_gpu_and_cpu_only_hosts():
+    import subprocess
+    import sys
+    bench = os.path.join(ROOT, "bench.py")
+    r = subprocess.run([sys.executable, bench, "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 2 and "ONE GPU" in r.stderr and r.stdout.strip() == ""
+    if not torch.cuda.is_available():
+        r = subprocess.run([sys.executable, bench], capture_output=True, text=True, timeout=120)
+        assert r.returncode == 1 and "no GPU" in r.stderr and r.stdout.strip() == ""
+
+
+def test_ttft_model_specs_match_the_named_architectures():
+    from pbs_attn_amd.ttft import MODELS
+    m = MODELS["llama31_8b"]
+    assert (m["hidden_size"], m["num_hidden_layers"], m["num_attention_heads"], m["num_key_value_heads"],
+            m["head_dim"], m["intermediate_size"], m["vocab_size"], m["rope_theta"]) == \
+        (4096, 32, 32, 8, 128, 14336, 128256, 500000.0)
+    q = MODELS["qwen25_7b"]
+    assert (q["num_attention_heads"], q["num_key_value_heads"], q["hidden_size"] // q["num_attention_heads"]) == (28, 4, 128)
