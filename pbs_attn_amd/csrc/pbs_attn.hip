@@ -25,9 +25,10 @@
 //     reference maximum: it is not updated per tile; a row sum of one tile above 2^14 triggers a
 //     uniform rescale (exact, all terms share the reference); an overflow marks the row and the
 //     whole workgroup redoes it without speculation.
-//   * careful tiles (the first tile of a row, tiles of the query block's own segment, and the redo
-//     pass): all of S first, exact running maximum, element mask "original key position > query
-//     position" in the own segment.
+//     Tiles of the query block's own segment run the same pipeline with the element mask "original
+//     key position > query position"; the tile's key positions travel to LDS with the tile.
+//   * careful tiles (the first tile of a row, own-segment tiles while some query has seen no key yet,
+//     and the redo pass): all of S first, exact running maximum, classic online softmax.
 #include "pbs_common.h"
 
 namespace {
@@ -38,6 +39,7 @@ constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
 constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
 constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096)
 constexpr uint32_t LDS_MISC = LDS_LIST + 8192;    // ints: [0] merged count, [1] redo flag, [16..528) scan
+constexpr uint32_t LDS_KPOS = LDS_MISC + 3072;    // 2 x 512 B: original key positions of the tile in flight
 constexpr uint32_t LDS_TOTAL = LDS_MISC + 4096;   // 143 360 bytes of the CU's 160 KB
 constexpr int PREFETCH_SLOTS = 3;                 // LDS fragment reads run this many slots ahead
 
@@ -93,11 +95,95 @@ __device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t l
   }
 }
 
+// the 128 original key positions of a tile (512 bytes): lanes 0..31 of wave 0, 16 bytes each
+__device__ __forceinline__ void stage_kpos_async(const int32_t* src, uint32_t lds_byte, int wave, int lane) {
+  if (wave == 0 && lane < 32) {
+    const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_byte);
+    const uint64_t src0 = (uint64_t)(uintptr_t)src;
+    const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
+    const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
+    const uint64_t base = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
+    const uint32_t off = (uint32_t)lane * 16u;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory");
+  }
+}
+
 __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const lds_u8*)(uintptr_t)byte_addr);
 }
 
 #define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
+
+
+// ---- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved, S of sub-tile s (s <= 3),
+// exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2); S and P are
+// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  MASKED tiles
+// (the query block's own segment) read the tile's original key positions from LDS, two per slot, and
+// zero the exponentials of keys that lie after the query.
+template <bool MASKED, int PF>
+__device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t (&koff)[8],
+                                          const uint32_t (&voff)[8], uint32_t bufx, float c_log2, float& m_ref,
+                                          float& l_part, bool& poisoned, int qpos, uint32_t kpos_lds, int gh) {
+  const float negm = -m_ref;
+  float rsum[4] = {0.f, 0.f, 0.f, 0.f};
+  f32x16 sbuf[2];
+  bf16x8 pbuf[2][2];
+  constexpr int R = PF + 1;
+  bf16x8 frk[R], frv[R];
+#pragma unroll
+  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf((koff[n & 7] ^ bufx) + (n >> 3) * 8192);
+#pragma clang loop unroll(full)
+  for (int n = 0; n < 48; ++n) {
+    const int step = n >> 3, t = n & 7;
+    {   // fragment reads for slot n + PF
+      const int m = n + PF, mstep = m >> 3, mt = m & 7;
+      if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff[mt] ^ bufx) + mstep * 8192);
+      if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff[2 * (mstep - 2) + (mt >> 2)] ^ bufx) + (mt & 3) * 8192);
+    }
+    if (step <= 3) {
+      const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
+      sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
+    }
+    if (step >= 2) o[t & 3] = PBS_MFMA(frv[n % R], pbuf[step & 1][t >> 2], o[t & 3]);
+    if (step >= 1 && step <= 4) {
+      const int sb = (step - 1) & 1, r = 2 * t;
+      float x0 = sbuf[sb][r], x1 = sbuf[sb][r + 1];
+      if (MASKED) {
+        // registers r, r + 1 of sub-tile ks hold keys 32 ks + 16 (a4 >> 1) + 8 gh + 4 (a4 & 1) + (r & 3), a4 = r >> 2
+        const int ks = step - 1, a4 = r >> 2;
+        const int key = 32 * ks + 16 * (a4 >> 1) + 4 * (a4 & 1) + (r & 3);
+        typedef __attribute__((ext_vector_type(2))) int i32x2;
+        const i32x2 kp = *reinterpret_cast<const __attribute__((address_space(3))) i32x2*>(
+            (const lds_u8*)(uintptr_t)(kpos_lds + (uint32_t)(key + 8 * gh) * 4));
+        if (kp.x > qpos) x0 = -INFINITY;
+        if (kp.y > qpos) x1 = -INFINITY;
+      }
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm));
+      rsum[t & 3] += e0;
+      rsum[(t + 2) & 3] += e1;
+      pbuf[sb][r >> 3][r & 7] = (__bf16)e0;
+      pbuf[sb][r >> 3][(r & 7) + 1] = (__bf16)e1;
+    }
+    __builtin_amdgcn_sched_barrier(0);
+  }
+  const float rs = (rsum[0] + rsum[1]) + (rsum[2] + rsum[3]);
+  l_part += rs;
+  // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
+  // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
+  if (__any(rs > 16384.0f)) {
+    const float big = fmaxf(rs, xhalf_f32(rs));
+    if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
+    const float m_new = (big > 16384.0f) ? m_ref + __builtin_amdgcn_logf(big) : m_ref;
+    const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
+    m_ref = m_new;
+    l_part *= alpha;
+#pragma unroll
+    for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+  }
+}
 
 __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // starts at LDS offset 0
@@ -194,12 +280,14 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     float m_ref = -INFINITY;   // reference maximum, identical in lanes j and j + 32
     float l_part = 0.f;        // row sum of this lane's half of the keys
     bool first = true, poisoned = false;
+    bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
 
     __syncthreads();   // list build / previous attempt are done with the tile buffers
     if (n_tiles > 0) {
       const int kb0 = mlist[0] & 0x3fff;
       stage_tile_async(pk + (int64_t)kb0 * BS * D, 0, wave, lane_off);
       stage_tile_async(pvt + (int64_t)kb0 * BS * D, LDS_V0, wave, lane_off);
+      stage_kpos_async(idx + (int64_t)kb0 * BS, LDS_KPOS, wave, lane);
     }
     for (int it = 0; it < n_tiles; ++it) {
       const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it]);
@@ -212,11 +300,15 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       if (has_next) {
         stage_tile_async(pk + (int64_t)kb_next * BS * D, bufx ^ 0x8000u, wave, lane_off);
         stage_tile_async(pvt + (int64_t)kb_next * BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+        stage_kpos_async(idx + (int64_t)kb_next * BS, LDS_KPOS + ((it & 1) ? 0u : 512u), wave, lane);
       }
       if (!(ent & use_bit) || !qb_valid) continue;
       const bool masked = kb >= own_first;
+      const uint32_t kpos_lds = LDS_KPOS + ((it & 1) ? 512u : 0u);
 
-      if (first || masked || careful_only) {
+      // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
+      // single key yet (its reference maximum is still -inf)
+      if (first || careful_only || (masked && !all_seen)) {
         // ---------------- careful tile
         first = false;
         f32x16 s[4];
@@ -261,6 +353,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
           }
         l_part = l_part * alpha + rs;
         m_ref = m_new;
+        all_seen = !__any(m_ref == -INFINITY);
         if (__any(alpha != 1.0f)) {
 #pragma unroll
           for (int dt = 0; dt < 4; ++dt)
@@ -278,57 +371,8 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
             for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff[2 * ks + u] ^ bufx) + dt * 8192), pf, o[dt]);
           }
       } else {
-        // ---------------- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved,
-        //   S of sub-tile s (s <= 3), exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2);
-        //   S and P are double-buffered by sub-tile parity.  One scheduling barrier per slot keeps the order.
-        const float negm = -m_ref;
-        float rsum[4] = {0.f, 0.f, 0.f, 0.f};
-        f32x16 sbuf[2];
-        bf16x8 pbuf[2][2];
-        constexpr int R = PREFETCH_SLOTS + 1;
-        bf16x8 frk[R], frv[R];
-#pragma unroll
-        for (int n = 0; n < PREFETCH_SLOTS; ++n) frk[n % R] = ldsf((koff[n & 7] ^ bufx) + (n >> 3) * 8192);
-#pragma clang loop unroll(full)
-        for (int n = 0; n < 48; ++n) {
-          const int step = n >> 3, t = n & 7;
-          {   // fragment reads for slot n + PREFETCH_SLOTS
-            const int m = n + PREFETCH_SLOTS, mstep = m >> 3, mt = m & 7;
-            if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff[mt] ^ bufx) + mstep * 8192);
-            if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff[2 * (mstep - 2) + (mt >> 2)] ^ bufx) + (mt & 3) * 8192);
-          }
-          if (step <= 3) {
-            const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
-            sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
-          }
-          if (step >= 2) o[t & 3] = PBS_MFMA(frv[n % R], pbuf[step & 1][t >> 2], o[t & 3]);
-          if (step >= 1 && step <= 4) {
-            const int sb = (step - 1) & 1, r = 2 * t;
-            const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sbuf[sb][r], c_log2, negm));
-            const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sbuf[sb][r + 1], c_log2, negm));
-            rsum[t & 3] += e0;
-            rsum[(t + 2) & 3] += e1;
-            pbuf[sb][r >> 3][r & 7] = (__bf16)e0;
-            pbuf[sb][r >> 3][(r & 7) + 1] = (__bf16)e1;
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        const float rs = (rsum[0] + rsum[1]) + (rsum[2] + rsum[3]);
-        l_part += rs;
-        // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
-        // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
-        if (__any(rs > 16384.0f)) {
-          const float big = fmaxf(rs, xhalf_f32(rs));
-          if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
-          const float m_new = (big > 16384.0f) ? m_ref + __builtin_amdgcn_logf(big) : m_ref;
-          const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-          m_ref = m_new;
-          l_part *= alpha;
-#pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-        }
+        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
+        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
       }
     }
     if (poisoned) misc[1] = 1;
