@@ -94,6 +94,23 @@ int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, 
 int pbs_unpermute(const void* o_perm, const int32_t* q_idx, void* out, int B, int H, int S, int head_dim,
                   int64_t o_sb, int64_t o_sh, int64_t o_ss, void* stream);
 
+/* key_indices[r, i] = i for every row: the order of a sequence that is not permuted
+ * (pbs_attn/src/permute_states.py:36-38). */
+int pbs_identity_indices(int32_t* key_indices, int rows, int S_pad, void* stream);
+
+/* The whole path in one call: key scoring, segment sort, gather, estimation, selection and sparse
+ * attention enqueued back to back on `stream`, intermediates in `workspace` (256-byte aligned,
+ * pbs_prefill_attn_workspace_bytes).  S <= segment_size gives plain causal attention, as the
+ * reference does.  Replaces pbs_attn/src/pbs.py:132-257 as a whole. */
+size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int S, int head_dim, int block_size, int segment_size);
+int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out, int B, int Hq, int Hkv, int S,
+                         int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                         int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                         int64_t o_sb, int64_t o_sh, int64_t o_ss, float threshold, const float* threshold_per_row,
+                         int threshold_is_int_one, int force_select_first_block, int query_pool_max,
+                         int key_pool_max, float softmax_scale, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
 #ifdef __cplusplus
 }
 #endif

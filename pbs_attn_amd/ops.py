@@ -162,6 +162,39 @@ def sparse_attn_fwd(q, perm_k, perm_vt, idx, csr_cols, csr_cnt, segment_size, so
     return out
 
 
+def prefill_attn_fwd(q, k, v, block_size, segment_size, threshold, force_select_first_block=True,
+                     query_pool_mode="mean", key_pool_mode="mean", softmax_scale=None):
+    """Every stage in one library call (pbs.py:132-257): one workspace allocation, one
+    host round trip.  Returns (B, Hq, S, D)."""
+    _check_bf16_cuda(q, k, v)
+    for mode, what in ((query_pool_mode, "query_pool_mode"), (key_pool_mode, "key_pool_mode")):
+        if mode not in ("mean", "max"):
+            raise ValueError(f"Invalid {what}: {mode}")
+    lib = _lib.load()
+    q, k, v = _rows16(q), _rows16(k), _rows16(v)
+    B, Hq, S, D = q.shape
+    Hkv = k.shape[1]
+    if softmax_scale is None:
+        softmax_scale = 1.0 / math.sqrt(D)
+    is_int_one = isinstance(threshold, int) and not isinstance(threshold, bool) and threshold == 1
+    thr_rows, thr = None, 0.0
+    if isinstance(threshold, torch.Tensor):
+        thr_rows = threshold.to(device=q.device, dtype=torch.float32).expand(B, Hq).contiguous()
+    elif not is_int_one:
+        thr = float(threshold)
+    out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
+    ws_bytes = lib.pbs_prefill_attn_workspace_bytes(B, Hq, S, D, block_size, segment_size)
+    ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.pbs_prefill_attn_fwd(
+        _ptr(q), _ptr(k), _ptr(v), _ptr(out), B, Hq, Hkv, S, D, block_size, segment_size,
+        q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+        v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
+        thr, _ptr(thr_rows), int(is_int_one), int(bool(force_select_first_block)),
+        int(query_pool_mode == "max"), int(key_pool_mode == "max"), softmax_scale,
+        _ptr(ws), ws.numel(), _stream()), "pbs_prefill_attn_fwd")
+    return out
+
+
 def unpermute(o_perm, q_idx=None, out=None):
     """out[b, h, q_idx[b, h, i]] = o_perm[b, h, i]; identity (no launch) when the
     queries were not permuted."""

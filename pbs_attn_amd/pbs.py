@@ -133,6 +133,12 @@ def permuted_block_sparse_attn_fwd(
         warnings.warn("use_triton=False: this build has a single implementation (HIP kernels); the flag is ignored")
         _warned_use_triton = True
 
+    if stage_timer is None:
+        # the whole path in one library call; the staged path below does the same work stage by
+        # stage so that a profiler hook can stamp each one
+        return ops.prefill_attn_fwd(query_states, key_states, value_states, block_size, segment_size, threshold,
+                                    force_select_first_block, query_pool_mode, key_pool_mode)
+
     if q_len <= segment_size:
         # pbs.py:175-182: plain causal attention.  Same kernel, one segment spanning the
         # sequence, identity order, every causal block visited.

@@ -332,3 +332,49 @@ def test_select_blocks_prefix_on_the_float32_rounding_boundary(dev):
         ref_sel, ref_fin = _oracle_selection(Pm, thr, idx_pad, nb, bps, False)
         sel, fin, _, _ = ops.select_blocks(Pm.to(dev), thr, idx_pad.to(dev), nb * 128, 128, bps * 128, False)
         assert torch.equal(sel.cpu(), ref_sel) and torch.equal(fin.cpu(), ref_fin), thr
+
+
+class _NullTimer:
+    def mark(self, name):
+        pass
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,seg,thr,kw", [
+    (1, 4, 2, 2048, 256, 0.9, {}),
+    (2, 3, 1, 1111, 256, 0.8, dict(query_pool_mode="max", key_pool_mode="max")),
+    (1, 2, 2, 1900, 512, "rows", dict(force_select_first_block=False)),
+    (1, 4, 4, 1024, 1024, 0.9, {}),
+    (1, 2, 1, 77, 256, 0.9, {}),
+    (1, 2, 2, 1536, 256, 1, {}),
+])
+def test_single_call_entry_point_equals_staged_path(dev, B, Hq, Hkv, S, seg, thr, kw):
+    # pbs_prefill_attn_fwd enqueues the same kernels on the same data as the stage-by-stage calls:
+    # the two outputs are bitwise equal
+    q, k, v = small_case(B, Hq, Hkv, S, seed=S + 1)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    if thr == "rows":
+        thr = torch.linspace(0.5, 0.95, B * Hq).view(B, Hq).to(dev)
+    assert P.stage_timer is None
+    one = P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, seg, thr, True, **kw)
+    P.stage_timer = _NullTimer()
+    try:
+        staged = P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, seg, thr, True, **kw)
+    finally:
+        P.stage_timer = None
+    assert torch.equal(one, staged)
+
+
+def test_single_call_entry_point_rejects_small_workspace(dev):
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    q, k, v = small_case(1, 2, 2, 512, seed=3)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out = torch.empty_like(qd)
+    need = lib.pbs_prefill_attn_workspace_bytes(1, 2, 512, 128, 128, 256)
+    assert need > 0
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    st = [t.stride(i) for t in (qd, kd, vd, out) for i in range(3)]
+    rc = lib.pbs_prefill_attn_fwd(qd.data_ptr(), kd.data_ptr(), vd.data_ptr(), out.data_ptr(), 1, 2, 2, 512, 128, 128, 256,
+                                  *st, 0.9, None, 0, 1, 0, 0, 128 ** -0.5, ws.data_ptr(), need - 256,
+                                  torch.cuda.current_stream().cuda_stream)
+    assert rc < 0 and b"workspace too small" in lib.pbs_last_error()
