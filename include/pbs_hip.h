@@ -31,7 +31,7 @@ const char* pbs_last_error(void);
  * softmax_k(bf16(bf16(q.k) / sqrt(D))) over the keys of the complete segments.
  * scores: (B, Hq, Sc) float32, Sc = (S / segment_size) * segment_size.
  * Replaces pbs_attn/src/permute_states.py:44-50. */
-size_t pbs_score_keys_workspace_bytes(int B, int Hq, int S, int segment_size);
+size_t pbs_score_keys_workspace_bytes(int B, int Hq, int Hkv, int S, int segment_size);
 int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
                    int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
                    int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream);
@@ -102,7 +102,8 @@ int pbs_identity_indices(int32_t* key_indices, int rows, int S_pad, void* stream
  * attention enqueued back to back on `stream`, intermediates in `workspace` (256-byte aligned,
  * pbs_prefill_attn_workspace_bytes).  S <= segment_size gives plain causal attention, as the
  * reference does.  Replaces pbs_attn/src/pbs.py:132-257 as a whole. */
-size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int S, int head_dim, int block_size, int segment_size);
+size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int Hkv, int S, int head_dim, int block_size,
+                                        int segment_size);
 int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out, int B, int Hq, int Hkv, int S,
                          int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
                          int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,

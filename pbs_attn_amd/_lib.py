@@ -13,7 +13,7 @@ _P, _I, _L, _F, _Z = c_void_p, c_int, c_int64, c_float, c_size_t
 SIGNATURES = {
     "pbs_abi_version": (c_int, []),
     "pbs_last_error": (c_char_p, []),
-    "pbs_score_keys_workspace_bytes": (_Z, [_I, _I, _I, _I]),
+    "pbs_score_keys_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "pbs_score_keys": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _Z, _P]),
     "pbs_segment_argsort": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "pbs_gather_kv": (c_int, [_P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _I, _P]),
@@ -24,7 +24,7 @@ SIGNATURES = {
     "pbs_sparse_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _F, _P]),
     "pbs_unpermute": (c_int, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
     "pbs_identity_indices": (c_int, [_P, _I, _I, _P]),
-    "pbs_prefill_attn_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I]),
+    "pbs_prefill_attn_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I, _I]),
     "pbs_prefill_attn_fwd": (c_int, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 12 +
                              [_F, _P, _I, _I, _I, _I, _F, _P, _Z, _P]),
 }

@@ -17,7 +17,7 @@ struct Layout {
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
-Layout make_layout(int B, int Hq, int S, int D, int block_size, int segment_size) {
+Layout make_layout(int B, int Hq, int Hkv, int S, int D, int block_size, int segment_size) {
   Layout L;
   const size_t rows = (size_t)B * Hq;
   const size_t nb = (size_t)(S + block_size - 1) / block_size, s_pad = nb * block_size;
@@ -25,7 +25,7 @@ Layout make_layout(int B, int Hq, int S, int D, int block_size, int segment_size
   size_t off = 0;
   auto take = [&](size_t bytes) { const size_t o = off; off = align256(off + bytes); return o; };
   L.scores = take(rows * sc * 4);
-  L.score_ws = take(pbs_score_keys_workspace_bytes(B, Hq, S, segment_size));
+  L.score_ws = take(pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size));
   L.idx = take(rows * s_pad * 4);
   L.perm_k = take(rows * s_pad * D * 2);
   L.perm_vt = take(rows * s_pad * D * 2);
@@ -49,10 +49,10 @@ extern "C" int pbs_identity_indices(int32_t* key_indices, int rows, int S_pad, v
   return pbs_check_launch("pbs_identity_indices");
 }
 
-extern "C" size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int S, int head_dim, int block_size, int segment_size) {
-  if (B <= 0 || Hq <= 0 || S <= 0 || head_dim <= 0 || block_size <= 0 || segment_size <= 0) return 0;
+extern "C" size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size) {
+  if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || S <= 0 || head_dim <= 0 || block_size <= 0 || segment_size <= 0) return 0;
   if (S <= segment_size) segment_size = (S + block_size - 1) / block_size * block_size;   // as pbs_prefill_attn_fwd
-  return make_layout(B, Hq, S, head_dim, block_size, segment_size).total;
+  return make_layout(B, Hq, Hkv, S, head_dim, block_size, segment_size).total;
 }
 
 extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out, int B, int Hq, int Hkv, int S,
@@ -72,7 +72,7 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
     segment_size = (S + block_size - 1) / block_size * block_size;
     threshold_is_int_one = 1;
   }
-  const Layout L = make_layout(B, Hq, S, head_dim, block_size, segment_size);
+  const Layout L = make_layout(B, Hq, Hkv, S, head_dim, block_size, segment_size);
   PBS_REQUIRE(workspace && workspace_bytes >= L.total, "pbs_prefill_attn_fwd: workspace too small (%zu < %zu bytes)",
               workspace_bytes, L.total);
   PBS_REQUIRE(((uintptr_t)workspace % 256) == 0, "pbs_prefill_attn_fwd: workspace must be 256-byte aligned");

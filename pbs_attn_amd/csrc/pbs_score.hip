@@ -4,7 +4,7 @@
 // Three launches, K is read twice and never re-materialised:
 //   (all exponentials are base 2 on logits pre-multiplied by log2(e))
 //   1. score_partial : per (head, key chunk) online (max, sum-exp) of every query row
-//   2. score_reduce  : fold the chunk partials into (row max, 1 / row sum)
+//   2. score_reduce  : fold the chunk partials into row max + log2(row sum)
 //   3. score_final   : recompute the logits and emit the per-key mean probability
 // Logits reproduce the rounding points of a bf16 matmul followed by a bf16
 // divide: fp32 accumulate -> bf16 -> / sqrt(D) -> bf16.
@@ -25,7 +25,7 @@ struct ScoreArgs {
   int64_t k_sb, k_sh, k_ss;
   float inv_sqrt_d;
   float* part;    // (B*Hq, nchunk, NQ, 2)
-  float* stats;   // (B*Hq, NQ, 2)  (max, 1/sum)
+  float* stats;   // (B*Hq, NQ)  row max + log2(row sum)
   float* scores;  // (B*Hq, Sc)
   int nchunk;
   int chunk_keys;
@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
   const int nwaves = blockDim.x >> 6;
   const uint16_t* kbase = a.k + b * a.k_sb + kvh * a.k_sh;
 
-  __shared__ float s_stats[4][NQ][2];
+  __shared__ float s_stats[4][NQ];   // per query row: max + log2(sum), so that p = exp2(logit - stat)
 
   for (int g0 = 0; g0 < G; g0 += nwaves) {
     const int g = g0 + wave;
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
     if (FINAL) {
       __syncthreads();
       if (active)
-        for (int i = lane; i < NQ * 2; i += 64) (&s_stats[wave][0][0])[i] = a.stats[(int64_t)bh * NQ * 2 + i];
+        for (int i = lane; i < NQ; i += 64) s_stats[wave][i] = a.stats[(int64_t)bh * NQ + i];
       __syncthreads();
     }
 
@@ -91,12 +91,23 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
     }
 
     if (active) {
+      // the next step's key rows are in flight while this step computes
+      bf16x8 kf_next[8];
+      {
+        const uint16_t* krow = kbase + (int64_t)(key_lo + j) * a.k_ss;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) kf_next[t] = load_frag(krow, t, half);
+      }
       for (int key0 = key_lo; key0 < key_hi; key0 += KEYS_PER_WAVE_STEP) {
         const int key = key0 + j;  // always < Sc: Sc is a multiple of 128
-        const uint16_t* krow = kbase + (int64_t)key * a.k_ss;
         bf16x8 kf[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) kf[t] = load_frag(krow, t, half);
+        for (int t = 0; t < 8; ++t) kf[t] = kf_next[t];
+        if (key0 + KEYS_PER_WAVE_STEP < key_hi) {
+          const uint16_t* krow = kbase + (int64_t)(key + KEYS_PER_WAVE_STEP) * a.k_ss;
+#pragma unroll
+          for (int t = 0; t < 8; ++t) kf_next[t] = load_frag(krow, t, half);
+        }
 
         if (!FINAL) {
           // S^T tile: rows = keys, column = query j of sub-tile qt
@@ -127,10 +138,12 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
 #pragma unroll
             for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[qt][t], kf[t], acc, 0, 0, 0);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const int qrow = 32 * qt + 8 * (r >> 2) + 4 * half + (r & 3);
-              const float mx = s_stats[wave][qrow][0], inv = s_stats[wave][qrow][1];
-              accp += __builtin_amdgcn_exp2f(logit_log2(acc[r], a.inv_sqrt_d) - mx) * inv;
+            for (int r4 = 0; r4 < 4; ++r4) {
+              const float4 st = *reinterpret_cast<const float4*>(&s_stats[wave][32 * qt + 8 * r4 + 4 * half]);
+              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 0], a.inv_sqrt_d) - st.x);
+              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 1], a.inv_sqrt_d) - st.y);
+              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 2], a.inv_sqrt_d) - st.z);
+              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 3], a.inv_sqrt_d) - st.w);
             }
           }
           accp += xhalf_f32(accp);
@@ -164,21 +177,29 @@ __global__ __launch_bounds__(NQ) void score_reduce_kernel(ScoreArgs a) {
     l = l * __builtin_amdgcn_exp2f(m - m_new) + lc * __builtin_amdgcn_exp2f(mc - m_new);
     m = m_new;
   }
-  a.stats[((int64_t)bh * NQ + qrow) * 2] = m;
-  a.stats[((int64_t)bh * NQ + qrow) * 2 + 1] = 1.0f / l;
+  a.stats[(int64_t)bh * NQ + qrow] = m + __builtin_amdgcn_logf(l);   // log base 2
 }
 
-// With one query head per KV head a workgroup is a single wave and takes a
-// quarter of the keys, so the launch still fills the chip.
-int chunk_keys_for(int G) { return G > 1 ? KEYS_PER_WG : KEYS_PER_WG / 4; }
 int chunks_for(int Sc, int chunk_keys) { return (Sc + chunk_keys - 1) / chunk_keys; }
+
+// Keys per workgroup.  With one query head per KV head a workgroup is a single wave and starts from a
+// quarter of the keys; short sequences get shorter chunks until the launch has enough workgroups to
+// fill the chip (each workgroup re-reads its heads' 128 queries, so chunks stay >= 64 keys).
+int chunk_keys_for(int B, int Hq, int Hkv, int Sc) {
+  const bool grouped = Hq / Hkv > 1;
+  int chunk = grouped ? KEYS_PER_WG : KEYS_PER_WG / 4;
+  const int64_t want = grouped ? 512 : 2048;
+  while (chunk > 64 && (int64_t)chunks_for(Sc, chunk) * B * Hkv < want) chunk /= 2;
+  return chunk;
+}
 
 }  // namespace
 
-extern "C" size_t pbs_score_keys_workspace_bytes(int B, int Hq, int S, int segment_size) {
-  if (segment_size <= 0) return 0;
+extern "C" size_t pbs_score_keys_workspace_bytes(int B, int Hq, int Hkv, int S, int segment_size) {
+  if (segment_size <= 0 || B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv) return 0;
   const int Sc = (S / segment_size) * segment_size;
-  return (size_t)B * Hq * ((size_t)chunks_for(Sc, KEYS_PER_WG / 4) + 1) * NQ * 2 * sizeof(float);
+  if (Sc == 0) return 0;
+  return (size_t)B * Hq * ((size_t)chunks_for(Sc, chunk_keys_for(B, Hq, Hkv, Sc)) + 1) * NQ * 2 * sizeof(float);
 }
 
 extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
@@ -195,7 +216,7 @@ extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B
   PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0, "pbs_score_keys: pointers must be 16-byte aligned");
   const int Sc = (S / segment_size) * segment_size;
   if (Sc == 0) return 0;
-  PBS_REQUIRE(workspace && workspace_bytes >= pbs_score_keys_workspace_bytes(B, Hq, S, segment_size),
+  PBS_REQUIRE(workspace && workspace_bytes >= pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size),
               "pbs_score_keys: workspace too small");
   ScoreArgs a;
   a.q = (const uint16_t*)q;
@@ -204,7 +225,7 @@ extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
   a.inv_sqrt_d = (float)(1.0 / sqrt((double)head_dim));
-  a.chunk_keys = chunk_keys_for(Hq / Hkv);
+  a.chunk_keys = chunk_keys_for(B, Hq, Hkv, Sc);
   a.nchunk = chunks_for(Sc, a.chunk_keys);
   a.part = (float*)workspace;
   a.stats = a.part + (size_t)B * Hq * a.nchunk * NQ * 2;

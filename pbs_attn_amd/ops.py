@@ -45,7 +45,7 @@ def score_keys(q, k, block_size, segment_size):
     Hkv = k.shape[1]
     Sc = (S // segment_size) * segment_size
     scores = torch.empty((B, Hq, Sc), dtype=torch.float32, device=q.device)
-    ws_bytes = lib.pbs_score_keys_workspace_bytes(B, Hq, S, segment_size)
+    ws_bytes = lib.pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size)
     ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
     _lib.check(lib.pbs_score_keys(_ptr(q), _ptr(k), _ptr(scores), B, Hq, Hkv, S, D, block_size, segment_size,
                                   q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
@@ -183,7 +183,7 @@ def prefill_attn_fwd(q, k, v, block_size, segment_size, threshold, force_select_
     elif not is_int_one:
         thr = float(threshold)
     out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
-    ws_bytes = lib.pbs_prefill_attn_workspace_bytes(B, Hq, S, D, block_size, segment_size)
+    ws_bytes = lib.pbs_prefill_attn_workspace_bytes(B, Hq, Hkv, S, D, block_size, segment_size)
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)
     _lib.check(lib.pbs_prefill_attn_fwd(
         _ptr(q), _ptr(k), _ptr(v), _ptr(out), B, Hq, Hkv, S, D, block_size, segment_size,

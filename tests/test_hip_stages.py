@@ -370,7 +370,7 @@ def test_single_call_entry_point_rejects_small_workspace(dev):
     q, k, v = small_case(1, 2, 2, 512, seed=3)
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     out = torch.empty_like(qd)
-    need = lib.pbs_prefill_attn_workspace_bytes(1, 2, 512, 128, 128, 256)
+    need = lib.pbs_prefill_attn_workspace_bytes(1, 2, 2, 512, 128, 128, 256)
     assert need > 0
     ws = torch.empty(need, dtype=torch.uint8, device=dev)
     st = [t.stride(i) for t in (qd, kd, vd, out) for i in range(3)]
