@@ -27,8 +27,8 @@
 //     whole workgroup redoes it without speculation.
 //     Tiles of the query block's own segment run the same pipeline with the element mask "original
 //     key position > query position"; the tile's key positions travel to LDS with the tile.
-//   * careful tiles (the first tile of a row, own-segment tiles while some query has seen no key yet,
-//     and the redo pass): all of S first, exact running maximum, classic online softmax.
+//   * careful tiles (a row that starts inside its own segment, own-segment tiles while some query has
+//     seen no key yet, and the redo pass): all of S first, exact running maximum, classic online softmax.
 #include "pbs_common.h"
 
 namespace {
@@ -207,54 +207,78 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   uint16_t* mlist = reinterpret_cast<uint16_t*>(smem + LDS_LIST);
   int* misc = reinterpret_cast<int*>(smem + LDS_MISC);
 
-  // ---- merged visit list of the two query blocks: entry = kb | use_first << 14 | use_second << 15
+  // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7.  Issued first so that the loads
+  // are in flight while the visit list is built.  Rows past the end of the sequence compute on the last
+  // row's values and are never stored.
+  bf16x8 qf[8];
   {
-    uint8_t* flags = smem;   // nb bytes; the tile area is free before the main loop
-    for (int i = tid; i < a.nb; i += 512) flags[i] = 0;
+    const uint16_t* qrow = a.q + b * a.q_sb + h * a.q_sh + (int64_t)min(qpos, a.S - 1) * a.q_ss;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(qrow + 16 * t + 8 * gh);
+  }
+
+  // ---- merged visit list of the two query blocks: entry = kb | use_first << 14 | use_second << 15.
+  // Counts and both column lists are fetched together (entries past a row's count are read and ignored).
+  {
+    uint8_t* flags0 = smem;          // nb bytes each; the tile area is free before the main loop
+    uint8_t* flags1 = smem + 4096;
+    const bool second = 2 * pair + 1 < a.nb;
+    const int32_t* l0 = a.cols + ((int64_t)bh * a.nb + 2 * pair) * a.nb;
+    const int32_t* l1 = l0 + (second ? a.nb : 0);
+    const int n0 = a.cnt[(int64_t)bh * a.nb + 2 * pair];
+    const int n1 = second ? a.cnt[(int64_t)bh * a.nb + 2 * pair + 1] : 0;
+    constexpr int MAX_PER = 4096 / 512;
+    int c0[MAX_PER], c1[MAX_PER];
+#pragma unroll
+    for (int u = 0; u < MAX_PER; ++u) {
+      const int i = tid + 512 * u;
+      c0[u] = i < a.nb ? l0[i] : 0;
+      c1[u] = i < a.nb ? l1[i] : 0;
+    }
+    for (int i = tid; i < a.nb; i += 512) {
+      flags0[i] = 0;
+      flags1[i] = 0;
+    }
     if (tid == 0) misc[1] = 0;
     __syncthreads();
-    const int n0 = a.cnt[(int64_t)bh * a.nb + 2 * pair];
-    const int32_t* l0 = a.cols + ((int64_t)bh * a.nb + 2 * pair) * a.nb;
-    for (int i = tid; i < n0; i += 512) flags[l0[i]] = 1;
-    __syncthreads();
-    if (2 * pair + 1 < a.nb) {
-      const int n1 = a.cnt[(int64_t)bh * a.nb + 2 * pair + 1];
-      const int32_t* l1 = l0 + a.nb;
-      for (int i = tid; i < n1; i += 512) flags[l1[i]] |= 2;
+#pragma unroll
+    for (int u = 0; u < MAX_PER; ++u) {
+      const int i = tid + 512 * u;
+      if (i < n0) flags0[c0[u]] = 1;
+      if (i < n1) flags1[c1[u]] = 2;
     }
     __syncthreads();
+    // compaction: thread t owns `per` consecutive key blocks; wave-level prefix, then wave totals
     const int per = (a.nb + 511) / 512;
     const int k0 = tid * per, k1 = min(k0 + per, a.nb);
     int c = 0;
-    for (int kb = k0; kb < k1; ++kb) c += flags[kb] ? 1 : 0;
-    int* scan = misc + 16;
-    scan[tid] = c;
-    __syncthreads();
-    for (int off = 1; off < 512; off <<= 1) {
-      const int v = tid >= off ? scan[tid - off] : 0;
-      __syncthreads();
-      scan[tid] += v;
-      __syncthreads();
+    for (int kb = k0; kb < k1; ++kb) c += (flags0[kb] | flags1[kb]) ? 1 : 0;
+    int incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
     }
-    int w = scan[tid] - c;
-    for (int kb = k0; kb < k1; ++kb)
-      if (flags[kb]) mlist[w++] = (uint16_t)(kb | (flags[kb] << 14));
-    if (tid == 511) misc[0] = scan[511];
+    int* wsum = misc + 16;
+    if (lane == 63) wsum[wave] = incl;
+    __syncthreads();
+    int w = incl - c, total = 0;
+#pragma unroll
+    for (int x = 0; x < 8; ++x) {
+      const int ws = wsum[x];
+      if (x < wave) w += ws;
+      total += ws;
+    }
+    for (int kb = k0; kb < k1; ++kb) {
+      const int f = flags0[kb] | flags1[kb];
+      if (f) mlist[w++] = (uint16_t)(kb | (f << 14));
+    }
+    if (tid == 0) misc[0] = total;
     __syncthreads();
   }
   const int n_tiles = misc[0];
   const int own_first = (qb / a.bps) * a.bps;
 
-  // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7
-  bf16x8 qf[8];
-  {
-    const uint16_t* qrow = a.q + b * a.q_sb + h * a.q_sh + (int64_t)min(qpos, a.S - 1) * a.q_ss;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      qf[t] = *reinterpret_cast<const bf16x8*>(qrow + 16 * t + 8 * gh);
-      if (qpos >= a.S) qf[t] = (bf16x8){0, 0, 0, 0, 0, 0, 0, 0};
-    }
-  }
   const uint16_t* pk = a.pk + (int64_t)bh * a.nb * BS * D;
   const uint16_t* pvt = a.pvt + (int64_t)bh * a.nb * BS * D;
   const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS;
@@ -308,7 +332,21 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
 
       // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
       // single key yet (its reference maximum is still -inf)
-      if (first || careful_only || (masked && !all_seen)) {
+      if (first && !masked && !careful_only) {
+        // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good
+        // enough reference to start the pipelined path (later keys move it up lazily)
+        first = false;
+        f32x16 s0 = (f32x16){0};
+#pragma unroll
+        for (int t = 0; t < 8; ++t) s0 = PBS_MFMA(ldsf(koff[t] ^ bufx), qf[t], s0);
+        float mx = s0[0];
+#pragma unroll
+        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
+        mx = fmaxf(mx, xhalf_f32(mx));
+        m_ref = mx * c_log2;
+        all_seen = true;
+        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
+      } else if (first || careful_only || (masked && !all_seen)) {
         // ---------------- careful tile
         first = false;
         f32x16 s[4];
