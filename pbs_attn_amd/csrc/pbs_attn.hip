@@ -191,13 +191,14 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   const int j = lane & 31, gh = lane >> 5;
   const int grp = wave >> 2, wq = wave & 3;
 
-  // workgroup -> (head, pair of query blocks): heads stay on one XCD (blockIdx % 8), long rows first
+  // workgroup -> (head, pair of query blocks): a head stays on one XCD (blockIdx % 8) and an XCD works
+  // through one head at a time, long rows first, so the workgroups resident on an XCD walk the same
+  // permuted K/V stream at about the same pace and share its tiles in that XCD's L2
   const int npair = (a.nb + 1) >> 1;
   const int w_id = blockIdx.x;
   const int xcd = w_id & 7, slot_id = w_id >> 3;
-  const int heads_per_xcd = (a.BH + 7) >> 3;
-  const int bh = (slot_id % heads_per_xcd) * 8 + xcd;
-  const int pair = npair - 1 - slot_id / heads_per_xcd;
+  const int bh = (slot_id / npair) * 8 + xcd;
+  const int pair = npair - 1 - slot_id % npair;
   if (bh >= a.BH) return;
   const int b = bh / a.Hq, h = bh % a.Hq;
   const int qb = 2 * pair + grp;
