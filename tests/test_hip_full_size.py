@@ -138,3 +138,25 @@ def test_late_dominant_keys_take_the_rare_paths(dev, gain, what):
     ref = _sdpa(q.float(), k.float(), v.float())
     assert torch.isfinite(out.float()).all(), what
     assert_attn_close(out, ref, what=what)
+
+
+def test_more_than_1024_blocks_per_sequence(dev):
+    # 1300 blocks (with a ragged tail and a trailing partial segment): the selection kernel for long rows
+    # and the attention kernel's list handling beyond 1024 entries
+    S, seg = 1300 * 128 - 37, 1024
+    q, k, v = make_qkv(1, 2, 1, S, 128, "span_heavy", seed=9, device=dev)
+    out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, seg, 1, True)
+    assert_attn_close(out, _sdpa(q, k, v), what="threshold=1 vs SDPA at 1300 blocks")
+    perm = P.apply_permutation(q, k, v, 128, seg)
+    sel = P.permuted_block_selection(q, perm, 128, seg, 0.9)
+    out = ops.sparse_attn_fwd(q, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+    idx = perm.key_indices[:, :, :S].long()
+    pk, pv = perm.permuted_keys().float(), perm.permuted_values().float()
+    pos = torch.arange(S, device=dev)
+    for qb in (9, 700, 1299):
+        rows = slice(qb * 128, min(qb * 128 + 128, S))
+        logits = q[:, :, rows].float() @ pk.transpose(-1, -2) / 128 ** 0.5
+        allowed = sel["final_mask"][:, :, qb][:, :, None, :].repeat_interleave(128, -1)[..., :S] \
+            & (idx[:, :, None, :] <= pos[rows].view(1, 1, -1, 1))
+        ref = torch.softmax(logits.masked_fill(~allowed, float("-inf")), -1) @ pv
+        assert_attn_close(out[:, :, rows], ref, what=f"q block {qb} of 1300")
