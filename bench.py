@@ -63,6 +63,37 @@ class StageTimer:
         return {k: sum(v) / len(v) for k, v in tot.items()}
 
 
+def mfma_ceiling(torch, iters=200000):
+    """What a loop of nothing but bf16 MFMAs sustains on this GPU right now, on all-zero operands and on
+    normally distributed ones (the rate depends on the values: the chip lowers its clock to stay inside its
+    power limit).  The second figure is the practical ceiling for a kernel fed with data like attention's."""
+    import ctypes
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    gen = torch.Generator(device="cpu").manual_seed(7)
+    pools = {"zeros": torch.zeros(65536, dtype=torch.bfloat16, device=dev),
+             "normal": torch.randn(65536, generator=gen).to(torch.bfloat16).to(dev)}
+    st = torch.cuda.current_stream().cuda_stream
+    out = {"unit": "TFLOP/s", "kernel": "v_mfma_f32_32x32x16_bf16 only, 256 workgroups x 8 waves"}
+    for name, pool in pools.items():
+        clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+        _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), 2000, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
+        torch.cuda.synchronize()
+        clocks.zero_()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), iters, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1)
+        c = clocks.tolist()
+        out[name] = lib.pbs_mfma_probe_flop(iters) / ms / 1e9
+        out[name + "_shader_clock_mhz"] = 100.0 * c[0] / max(1, c[1])
+    return out
+
+
 def cpu_baseline(cfg, q, k, v, seconds_budget=20.0):
     """The reference's torch CPU path (restated in oracle/) on the SAME workload,
     bounded to whole query heads: head after head until `seconds_budget` is spent
@@ -112,7 +143,7 @@ def dense_sdpa_ms(torch, q, k, v, reps=3):
         return None
 
 
-def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=True):
+def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=True, with_zero_operands=False):
     from pbs_attn_amd import pbs as P
     from pbs_attn_amd.synth import make_workload
     dev = torch.device("cuda:0")
@@ -164,6 +195,21 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
         "gather": gather_b / (stages["gather"] * 1e-3) / 1e9,
         "estimate": est_b / (stages["estimate"] * 1e-3) / 1e9 if "estimate" in stages else None,
     }
+    if with_zero_operands:
+        # the same launch (same visit lists, same schedule) on all-zero Q, K, V: what the kernel's schedule
+        # delivers when the matrix cores draw the least power
+        from pbs_attn_amd import ops
+        zq, zk, zv = torch.zeros_like(q), torch.zeros_like(perm.perm_k), torch.zeros_like(perm.perm_vt)
+        zargs = (zq, zk, zv, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+        ops.sparse_attn_fwd(*zargs)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(2):
+            ops.sparse_attn_fwd(*zargs)
+        e1.record()
+        torch.cuda.synchronize()
+        res["attn_ms_zero_operands"] = e0.elapsed_time(e1) / 2
+        del zq, zk, zv
     if with_dense:
         res["dense_sdpa_ms"] = dense_sdpa_ms(torch, q, k, v)
         # the build's own kernel on the full causal mask (every candidate selected, one block per segment)
@@ -238,6 +284,7 @@ def main():
     ap.add_argument("--kind", default=None, help="override the input generator, e.g. strong_heavy")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-dense", action="store_true")
+    ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only ceiling measurement")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
     ap.add_argument("--report", default=None, metavar="FILE.md",
                     help="run every single-layer configuration and the sweeps, write a markdown table, and exit")
@@ -270,7 +317,7 @@ def main():
     if args.kind:
         overrides["kind"] = args.kind
     res, inputs = run_workload(torch, args.workload, args.steps, args.warmup, overrides=overrides,
-                               with_dense=not args.no_dense)
+                               with_dense=not args.no_dense, with_zero_operands=not args.no_mfma_probe)
     log("[bench] " + json.dumps(res))
     if args.traffic_calibration:
         cfg, q = inputs[0], inputs[1]
@@ -305,6 +352,12 @@ def main():
         "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
         "speedup_vs_dense_sdpa": res.get("speedup_vs_dense_sdpa"),
     }
+    if not args.no_mfma_probe:
+        # context for roofline.frac: `peak` stays the published figure, this is what the matrix cores
+        # sustain on this GPU on their own
+        line["mfma_ceiling"] = mfma_ceiling(torch)
+        line["roofline"]["frac_of_measured_ceiling"] = achieved / line["mfma_ceiling"]["normal"]
+        line["roofline"]["kernel_ms_zero_operands"] = res["attn_ms_zero_operands"]
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(*inputs, seconds_budget=args.cpu_seconds)
     print(json.dumps(line), flush=True)

@@ -112,6 +112,14 @@ int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out,
                          int key_pool_max, float softmax_scale, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* Measurement aid with no counterpart in the reference: `iters` x 8 v_mfma_f32_32x32x16_bf16 per wave on
+ * 256 workgroups of 8 waves, operands taken from `operands` (65536 bf16 values of the caller's choice: the
+ * sustained rate depends on the values).  `sink` takes 256 * 512 floats, `clocks` (two 64-bit counters the
+ * caller zeroes) accumulates shader-clock and 100 MHz ticks over the workgroups; time the launch with
+ * events.  pbs_mfma_probe_flop gives the FLOP count of one launch. */
+int pbs_mfma_probe(const void* operands, int iters, float* sink, unsigned long long* clocks, void* stream);
+double pbs_mfma_probe_flop(int iters);
+
 #ifdef __cplusplus
 }
 #endif

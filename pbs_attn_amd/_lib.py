@@ -23,6 +23,8 @@ SIGNATURES = {
     "pbs_select_blocks": (c_int, [_P, _P, _F, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _Z, _P]),
     "pbs_sparse_attn_fwd": (c_int, [_P, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _F, _P]),
     "pbs_unpermute": (c_int, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
+    "pbs_mfma_probe": (c_int, [_P, _I, _P, _P, _P]),
+    "pbs_mfma_probe_flop": (ctypes.c_double, [_I]),
     "pbs_identity_indices": (c_int, [_P, _I, _I, _P]),
     "pbs_prefill_attn_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I, _I]),
     "pbs_prefill_attn_fwd": (c_int, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 12 +
