@@ -243,7 +243,7 @@ def density_without_permutation(torch, cfg, q, k, v):
 
 
 def run_report(torch, path, steps, warmup):
-    """Every BASELINE.json single-layer configuration + sweeps, written as a markdown table."""
+    """Every single-layer benchmark configuration + sweeps, written as a markdown table."""
     runs = [("cfg0", {}), ("cfg1", {})]
     runs += [("cfg1", {"segment": sg, "threshold": th}) for sg in (256, 1024) for th in (0.8, 0.9, 0.95)
              if not (sg == 256 and th == 0.9)]

@@ -17,7 +17,7 @@ import sys
 import time
 
 MODELS = {
-    # Llama-3.1-8B architecture (BASELINE.json config 4)
+    # Llama-3.1-8B architecture (the 64k time-to-first-token configuration)
     "llama31_8b": dict(family="llama", hidden_size=4096, intermediate_size=14336, num_hidden_layers=32,
                        num_attention_heads=32, num_key_value_heads=8, head_dim=128, vocab_size=128256,
                        rms_norm_eps=1e-5, rope_theta=500000.0, max_position_embeddings=131072),
