@@ -35,16 +35,21 @@ __device__ __forceinline__ bf16x8 load_frag(const uint16_t* row_ptr, int t, int 
   return *reinterpret_cast<const bf16x8*>(row_ptr + 16 * t + 8 * half);
 }
 
-// fp32 accumulator -> the bf16 logit a bf16 matmul followed by a bf16 divide by sqrt(D) yields, times
-// log2(e): round to bf16, scale (multiplication by the reciprocal; it differs from the true quotient by
-// at most one fp32 ulp, which survives the second bf16 rounding only for values within 2^-16 of a tie),
-// round to bf16.  Hardware conversions (round to nearest even).
-__device__ __forceinline__ float hw_round_bf16(float x) {
-  return bf16_bits_to_f32((uint32_t)__builtin_bit_cast(uint16_t, (__bf16)x));
+// fp32 accumulator -> the bf16 logit a bf16 matmul followed by a bf16 divide by sqrt(D) yields: round to
+// bf16, scale (multiplication by the reciprocal; it differs from the true quotient by at most one fp32 ulp,
+// which survives the second bf16 rounding only for values within 2^-16 of a tie), round to bf16.
+// Hardware conversions (round to nearest even), two values per conversion instruction.
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+__device__ __forceinline__ f32x2 hw_round_bf16x2(f32x2 x) {
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+  return (f32x2){__builtin_bit_cast(float, packed << 16), __builtin_bit_cast(float, packed & 0xffff0000u)};
 }
-__device__ __forceinline__ float logit_log2(float acc, float inv_sqrt_d) {
-  return hw_round_bf16(hw_round_bf16(acc) * inv_sqrt_d) * 1.4426950408889634f;
+__device__ __forceinline__ f32x2 logit2(float acc0, float acc1, float inv_sqrt_d) {
+  const f32x2 r = hw_round_bf16x2((f32x2){acc0, acc1});
+  return hw_round_bf16x2((f32x2){r.x * inv_sqrt_d, r.y * inv_sqrt_d});
 }
+constexpr float LOG2E = 1.4426950408889634f;
 
 // One wave per query head of the KV group; the four waves of a workgroup walk
 // the same key chunk so K comes out of the CU's L1 after the first wave.
@@ -116,16 +121,18 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
             f32x16 acc = {0};
 #pragma unroll
             for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[t], qf[qt][t], acc, 0, 0, 0);
-            float v[16], mx = -INFINITY;
+            float v[16], mx = -INFINITY;   // logits before the log2(e) factor
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              v[r] = logit_log2(acc[r], a.inv_sqrt_d);
-              mx = fmaxf(mx, v[r]);
+            for (int r = 0; r < 16; r += 2) {
+              const f32x2 l2 = logit2(acc[r], acc[r + 1], a.inv_sqrt_d);
+              v[r] = l2.x;
+              v[r + 1] = l2.y;
+              mx = fmaxf(fmaxf(mx, l2.x), l2.y);
             }
-            const float m_new = fmaxf(m_run[qt], mx);
+            const float m_new = fmaxf(m_run[qt], mx * LOG2E);
             float sum = 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(v[r] - m_new);
+            for (int r = 0; r < 16; ++r) sum += __builtin_amdgcn_exp2f(__builtin_fmaf(v[r], LOG2E, -m_new));
             l_run[qt] = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + sum;
             m_run[qt] = m_new;
           }
@@ -140,10 +147,12 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
               const float4 st = *reinterpret_cast<const float4*>(&s_stats[wave][32 * qt + 8 * r4 + 4 * half]);
-              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 0], a.inv_sqrt_d) - st.x);
-              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 1], a.inv_sqrt_d) - st.y);
-              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 2], a.inv_sqrt_d) - st.z);
-              accp += __builtin_amdgcn_exp2f(logit_log2(acc[4 * r4 + 3], a.inv_sqrt_d) - st.w);
+              const f32x2 la = logit2(acc[4 * r4 + 0], acc[4 * r4 + 1], a.inv_sqrt_d);
+              const f32x2 lb = logit2(acc[4 * r4 + 2], acc[4 * r4 + 3], a.inv_sqrt_d);
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.x, LOG2E, -st.x));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.y, LOG2E, -st.y));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.x, LOG2E, -st.z));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.y, LOG2E, -st.w));
             }
           }
           accp += xhalf_f32(accp);

@@ -29,13 +29,21 @@ struct SelectArgs {
   int32_t* csr_cnt;        // (rows, nb)
 };
 
-__global__ __launch_bounds__(1024) void first_token_block_kernel(const int32_t* idx, int32_t* first_blk, int S_pad, int bs) {
+// Block that holds original key 0.  A segment-wise permutation keeps it inside the first segment, so that
+// part of the row is searched first; the rest only if it is not there (any index layout stays correct).
+__global__ __launch_bounds__(1024) void first_token_block_kernel(const int32_t* idx, int32_t* first_blk, int S_pad, int bs,
+                                                                 int first_span) {
   __shared__ int found;
   if (threadIdx.x == 0) found = -1;
   __syncthreads();
   const int32_t* row = idx + (int64_t)blockIdx.x * S_pad;
-  for (int i = threadIdx.x; i < S_pad; i += blockDim.x)
+  for (int i = threadIdx.x; i < first_span; i += blockDim.x)
     if (row[i] == 0) atomicMax(&found, i / bs);
+  __syncthreads();
+  if (found < 0) {
+    for (int i = first_span + threadIdx.x; i < S_pad; i += blockDim.x)
+      if (row[i] == 0) atomicMax(&found, i / bs);
+  }
   __syncthreads();
   if (threadIdx.x == 0) first_blk[blockIdx.x] = found;
 }
@@ -382,7 +390,8 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   a.sel_mask = sel_mask; a.final_mask = final_mask; a.csr_cols = csr_cols; a.csr_cnt = csr_cnt;
   hipStream_t st = (hipStream_t)stream;
   if (force_select_first_block)
-    hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size);
+    hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size,
+                       min(segment_size, nb * block_size));
   if (nb <= 1024) {
     // one wave per row, four rows per workgroup
     const int total = rows * nb;
