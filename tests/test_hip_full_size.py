@@ -140,6 +140,31 @@ def test_late_dominant_keys_take_the_rare_paths(dev, gain, what):
     assert_attn_close(out, ref, what=what)
 
 
+@pytest.mark.parametrize("gain,what", [(3.0, "lazy rescale inside the first tile"), (12.0, "many octaves inside the first tile"),
+                                       (60.0, "overflow inside the first tile -> redo")])
+def test_first_tile_reference_from_its_first_keys(dev, gain, what):
+    # the first tile of a row takes its reference maximum from its first 32 keys only; keys 40..127 of
+    # that tile are far stronger here (identity key order is forced through injected scores)
+    S, seg = 2048, 256
+    g = torch.Generator().manual_seed(11)
+    q = torch.randn((1, 2, S, 128), generator=g)
+    k = torch.randn((1, 2, S, 128), generator=g)
+    v = torch.randn((1, 2, S, 128), generator=g)
+    u = torch.zeros(128)
+    u[3] = 1.0
+    q = q + 4.0 * u
+    k[:, :, 40:128] += gain * 4.0 * u
+    q, k, v = (t.to(torch.bfloat16).to(dev) for t in (q, k, v))
+    scores = -torch.arange(S, device=dev, dtype=torch.float32).view(1, 1, S).expand(1, 2, S).contiguous()
+    perm = P.apply_permutation(q, k, v, 128, seg, scores=scores)
+    assert torch.equal(perm.key_indices[0, 0, :S].cpu(), torch.arange(S, dtype=torch.int32))
+    sel = P.permuted_block_selection(q, perm, 128, seg, 1, want_masks=False)
+    out = ops.sparse_attn_fwd(q, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+    ref = _sdpa(q.float(), k.float(), v.float())
+    assert torch.isfinite(out.float()).all(), what
+    assert_attn_close(out, ref, what=what)
+
+
 def test_more_than_1024_blocks_per_sequence(dev):
     # 1300 blocks (with a ragged tail and a trailing partial segment): the selection kernel for long rows
     # and the attention kernel's list handling beyond 1024 entries
