@@ -94,6 +94,18 @@ def mfma_ceiling(torch, iters=200000):
     return out
 
 
+def block_pair_counts(csr_cnt, B, Hq, nb, bps):
+    """(executed, reference) numbers of 128 x 128 tiles of one launch.  executed = what the HIP kernel
+    multiplies: the selected blocks of earlier segments plus the causal part of the own segment (blocks
+    first-of-segment .. query block, read in original key order).  reference = the tiles the reference's
+    kernel visits for the same masks: the same selected blocks plus EVERY block of the own segment (in
+    permuted order a block of the segment can hold visible keys wherever it lies)."""
+    earlier = int(csr_cnt.sum().item())
+    own_exec = sum(qb - (qb // bps) * bps + 1 for qb in range(nb))
+    own_all = sum(min((qb // bps) * bps + bps, nb) - (qb // bps) * bps for qb in range(nb))
+    return earlier + B * Hq * own_exec, earlier + B * Hq * own_all
+
+
 def cpu_baseline(cfg, q, k, v, seconds_budget=20.0):
     """The reference's torch CPU path (restated in oracle/) on the SAME workload,
     bounded to whole query heads: head after head until `seconds_budget` is spent
@@ -172,7 +184,7 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     # visited block pairs of this input (one extra selection pass, outside the timed region)
     perm = P.apply_permutation(q, k, v, bs, seg)
     sel = P.permuted_block_selection(q, perm, bs, seg, thr, want_masks=False)
-    n_vis = int(sel["csr_cnt"].sum().item())
+    n_vis, n_ref = block_pair_counts(sel["csr_cnt"], B, Hq, nb, seg // bs)
     causal_pairs = B * Hq * nb * (nb + 1) // 2
     flops = n_vis * FLOP_PER_BLOCK_PAIR
     attn_ms = stages["sparse_attn"]
@@ -180,6 +192,7 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
         "workload": name, "B": B, "Hq": Hq, "Hkv": Hkv, "S": S, "D": D, "block": bs, "segment": seg,
         "threshold": thr, "generator": cfg["kind"], "seed": seed,
         "ms_per_step": wall_ms, "stage_ms": stages, "visited_block_pairs": n_vis,
+        "reference_block_pairs": n_ref,
         "density_vs_causal": n_vis / causal_pairs,
         "effective_tflops_pipeline": flops / (wall_ms * 1e-3) / 1e12,
         "effective_tflops_attn_kernel": flops / (attn_ms * 1e-3) / 1e12,
@@ -200,7 +213,7 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
         # delivers when the matrix cores draw the least power
         from pbs_attn_amd import ops
         zq, zk, zv = torch.zeros_like(q), torch.zeros_like(perm.perm_k), torch.zeros_like(perm.perm_vt)
-        zargs = (zq, zk, zv, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+        zargs = (zq, zk, zv, torch.zeros_like(k), torch.zeros_like(perm.orig_vt), sel["csr_cols"], sel["csr_cnt"], seg)
         ops.sparse_attn_fwd(*zargs)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -239,7 +252,7 @@ def density_without_permutation(torch, cfg, q, k, v):
     perm = P.apply_permutation(q, k, v, bs, seg, scores=scores)
     sel = P.permuted_block_selection(q, perm, bs, seg, thr, want_masks=False)
     nb = (S + bs - 1) // bs
-    return int(sel["csr_cnt"].sum().item()) / (B * Hq * nb * (nb + 1) // 2)
+    return block_pair_counts(sel["csr_cnt"], B, Hq, nb, seg // bs)[0] / (B * Hq * nb * (nb + 1) // 2)
 
 
 def run_report(torch, path, steps, warmup):
@@ -340,7 +353,8 @@ def main():
                                f"Hkv={res['Hkv']} D={res['D']} S={res['S']}, block {res['block']}, segment "
                                f"{res['segment']}, threshold {res['threshold']}, generator {res['generator']} seed {res['seed']}",
                    "density_vs_causal": res["density_vs_causal"],
-                   "visited_block_pairs": res["visited_block_pairs"]},
+                   "visited_block_pairs": res["visited_block_pairs"],
+                   "reference_block_pairs": res["reference_block_pairs"]},
         "roofline": {"bound": "mfma", "kernel": "sparse_attn_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
                      "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, args.kind, res["segment"], res["threshold"])),

@@ -46,11 +46,14 @@ int pbs_segment_argsort(const float* scores, int32_t* key_indices, int rows, int
 
 /* Gather K and V into permuted order and pool the permuted key blocks.
  * perm_k: (B, Hq, nb*128, 128) rows past S zero; perm_vt: (B, Hq, nb, 128, 128)
- * holding each V block transposed [d][key]; pooled_k: (B, Hq, nb, 128) bf16.
+ * holding each V block transposed [d][key]; pooled_k: (B, Hq, nb, 128) bf16;
+ * orig_vt (may be null): (B, Hkv, nb, 128, 128), the V blocks in ORIGINAL key order,
+ * transposed the same way and zero past S -- the attention kernel reads a query
+ * block's own segment un-permuted, where the causal mask is a plain triangle.
  * Replaces pbs_attn/src/permute_states.py:59-69, pbs_attn/src/pbs.py:213-215,
  * the key padding of pbs.py:78-79 and the key pooling of pbs_attn/src/utils.py:24-29. */
 int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
-                  void* pooled_k, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
+                  void* pooled_k, void* orig_vt, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
                   int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
                   void* stream);
 
@@ -71,7 +74,9 @@ int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* 
  * `threshold` when non-null; threshold_is_int_one selects every candidate.
  * sel_mask = selected | first-token block; final_mask = sel_mask | own segment
  * (both (rows, nb, nb) bytes, either may be null); csr_cols (rows, nb, nb) /
- * csr_cnt (rows, nb): ascending key blocks the attention kernel visits.
+ * csr_cnt (rows, nb): the ascending key blocks of sel_mask that lie in segments
+ * strictly before the query block's -- the permuted tiles the attention kernel
+ * visits (it adds the causal part of the query block's own segment itself).
  * Replaces pbs_attn/src/utils.py:38-86 and pbs_attn/src/pbs.py:10-25,119-127,209. */
 size_t pbs_select_blocks_workspace_bytes(int rows);
 int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
@@ -79,14 +84,20 @@ int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per
                       int S, int block_size, int segment_size, uint8_t* sel_mask, uint8_t* final_mask,
                       int32_t* csr_cols, int32_t* csr_cnt, void* workspace, size_t workspace_bytes, void* stream);
 
-/* Block-sparse flash-attention forward over the permuted K / transposed V tiles.
+/* Block-sparse flash-attention forward.  Query block qb attends to the permuted K /
+ * transposed V tiles listed in csr_cols (earlier segments, no element mask) and to
+ * its own segment: blocks first-of-segment .. qb of the ORIGINAL k (B, Hkv, S, 128,
+ * caller's strides) and orig_vt, with the causal triangle on block qb.  The keys a
+ * query sees are exactly those of the reference's final mask and element mask
+ * (a segment's permuted blocks hold the same keys as its original blocks).
  * out: (B, Hq, S, 128) bf16 with its own strides, original query order.
  * Replaces pbs_attn/src/kernels/permuted_block_sparse_attention.py:134-311
  * (launch at pbs_attn/src/pbs.py:220-246). */
-int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const int32_t* key_indices,
-                        const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int S,
+int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+                        const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
                         int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                        int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale, void* stream);
+                        int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                        float softmax_scale, void* stream);
 
 /* out[b,h,q_idx[b,h,i],:] = o_perm[b,h,i,:] (o_perm contiguous).  q_idx null with
  * o_perm == out is the identity fast path (no launch): the reference does not

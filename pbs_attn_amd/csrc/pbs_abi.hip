@@ -1,5 +1,6 @@
 // Error reporting, version query and the output un-permutation of the C ABI.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <stdarg.h>
 #include <stdio.h>
 

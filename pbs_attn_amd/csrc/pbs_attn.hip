@@ -30,6 +30,7 @@
 //   * careful tiles (a row that starts inside its own segment, own-segment tiles while some query has
 //     seen no key yet, and the redo pass): all of S first, exact running maximum, classic online softmax.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
 
@@ -37,22 +38,25 @@ constexpr int D = 128;
 constexpr int BS = 128;
 constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
 constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
-constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096)
-constexpr uint32_t LDS_MISC = LDS_LIST + 8192;    // ints: [0] merged count, [1] redo flag, [16..528) scan
-constexpr uint32_t LDS_KPOS = LDS_MISC + 3072;    // 2 x 512 B: original key positions of the tile in flight
-constexpr uint32_t LDS_TOTAL = LDS_MISC + 4096;   // 143 360 bytes of the CU's 160 KB
+constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096 + 257)
+constexpr uint32_t LDS_MISC = LDS_LIST + 10240;   // ints: [0] merged count, [1] redo flag, [16..24) wave totals
+constexpr uint32_t LDS_TOTAL = LDS_MISC + 1024;   // 142 336 bytes of the CU's 160 KB
+constexpr uint32_t ENT_KB = 0x1fffu;              // visit-list entry: key block ...
+constexpr uint32_t ENT_ORIG = 0x2000u;            // ... | tile of the un-permuted K / V (own segment) | use bits 14, 15
 constexpr int PREFETCH_SLOTS = 3;                 // LDS fragment reads run this many slots ahead
 
 struct AttnArgs {
   const uint16_t* q;
-  const uint16_t* pk;    // (B*Hq, nb*128, 128)
-  const uint16_t* pvt;   // (B*Hq, nb, 128, 128)
-  const int32_t* idx;    // (B*Hq, nb*128)
+  const uint16_t* pk;    // (B*Hq, nb*128, 128)  permuted K
+  const uint16_t* pvt;   // (B*Hq, nb, 128, 128) permuted V blocks, transposed
+  const uint16_t* k;     // original K at the KV heads, caller's strides
+  const uint16_t* ovt;   // (B*Hkv, nb, 128, 128) original-order V blocks, transposed
   const int32_t* cols;   // (B*Hq, nb, nb)
   const int32_t* cnt;    // (B*Hq, nb)
   uint16_t* o;
-  int BH, Hq, S, nb, bps;
-  int64_t q_sb, q_sh, q_ss, o_sb, o_sh, o_ss;
+  int BH, Hq, Hkv, S, nb, bps;
+  uint32_t k_ss;   // key row stride in elements (< 2^22)
+  int64_t q_sb, q_sh, q_ss, k_sb, k_sh, o_sb, o_sh, o_ss;
   float scale_log2;
 };
 
@@ -95,16 +99,37 @@ __device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t l
   }
 }
 
-// the 128 original key positions of a tile (512 bytes): lanes 0..31 of wave 0, 16 bytes each
-__device__ __forceinline__ void stage_kpos_async(const int32_t* src, uint32_t lds_byte, int wave, int lane) {
-  if (wave == 0 && lane < 32) {
-    const uint32_t m0v = (uint32_t)__builtin_amdgcn_readfirstlane((int)lds_byte);
-    const uint64_t src0 = (uint64_t)(uintptr_t)src;
-    const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
-    const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
-    const uint64_t base = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
-    const uint32_t off = (uint32_t)lane * 16u;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(off), "s"(base) : "memory");
+// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride (same LDS layout and swizzle).  Rows
+// past the end of the sequence re-read the last valid row: their keys lie after every query and are masked.
+__device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t row_stride, int rows_valid, uint32_t lds_byte,
+                                                  int wave, int lane) {
+  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + wave * 1024));
+  const uint64_t src0 = (uint64_t)(uintptr_t)src;
+  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
+  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
+  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
+  // lane l of wave w fetches chunk (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4); offsets fit 32 bits
+  // (row stride < 2^22 elements, checked on the host)
+  const uint32_t r0 = (uint32_t)(4 * wave + (lane >> 4));
+  const uint32_t c16 = (uint32_t)(((lane & 15) ^ (r0 & 15)) * 16);
+  if (rows_valid >= BS) {
+    const uint32_t voff = r0 * row_stride * 2u + c16;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const uint64_t base = srcu + (uint64_t)n * (64u * row_stride);
+      const uint32_t m0v = lds0 + n * 8192;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base)
+                   : "memory");
+    }
+  } else {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const uint32_t row = min(r0 + 32u * n, (uint32_t)(rows_valid - 1));
+      const uint32_t voff = row * row_stride * 2u + c16;
+      const uint32_t m0v = lds0 + n * 8192;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu)
+                   : "memory");
+    }
   }
 }
 
@@ -117,13 +142,16 @@ __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
 
 // ---- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved, S of sub-tile s (s <= 3),
 // exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2); S and P are
-// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  MASKED tiles
-// (the query block's own segment) read the tile's original key positions from LDS, two per slot, and
-// zero the exponentials of keys that lie after the query.
+// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  The MASKED tile
+// (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
+// query: key-in-tile > query-in-block, an arithmetic test (`qrel8` = query-in-block - 8 * lane half).
 template <bool MASKED, int PF>
 __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t (&koff)[8],
                                           const uint32_t (&voff)[8], uint32_t bufx, float c_log2, float& m_ref,
-                                          float& l_part, bool& poisoned, int qpos, uint32_t kpos_lds, int gh) {
+                                          float& l_part, bool& poisoned, int qrel8) {
+  // opaque per call: the 128 mask compares of a diagonal tile depend only on the lane, and hoisted out of
+  // the tile loop they would each pin a 64-bit scalar mask
+  if (MASKED) asm volatile("" : "+v"(qrel8));
   const float negm = -m_ref;
   float rsum[4] = {0.f, 0.f, 0.f, 0.f};
   f32x16 sbuf[2];
@@ -152,11 +180,8 @@ __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8],
         // registers r, r + 1 of sub-tile ks hold keys 32 ks + 16 (a4 >> 1) + 8 gh + 4 (a4 & 1) + (r & 3), a4 = r >> 2
         const int ks = step - 1, a4 = r >> 2;
         const int key = 32 * ks + 16 * (a4 >> 1) + 4 * (a4 & 1) + (r & 3);
-        typedef __attribute__((ext_vector_type(2))) int i32x2;
-        const i32x2 kp = *reinterpret_cast<const __attribute__((address_space(3))) i32x2*>(
-            (const lds_u8*)(uintptr_t)(kpos_lds + (uint32_t)(key + 8 * gh) * 4));
-        if (kp.x > qpos) x0 = -INFINITY;
-        if (kp.y > qpos) x1 = -INFINITY;
+        if (key > qrel8) x0 = -INFINITY;
+        if (key + 1 > qrel8) x1 = -INFINITY;
       }
       const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm));
       const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm));
@@ -274,15 +299,26 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       const int f = flags0[kb] | flags1[kb];
       if (f) mlist[w++] = (uint16_t)(kb | (f << 14));
     }
-    if (tid == 0) misc[0] = total;
+    // then the own segments in ORIGINAL key order: blocks first-of-segment .. query block (causal), the
+    // same for both query blocks where they share a segment
+    const int qb0 = 2 * pair, qb1 = second ? qb0 + 1 : qb0;
+    const int sf0 = (qb0 / a.bps) * a.bps, sf1 = (qb1 / a.bps) * a.bps;
+    const int n_own = qb1 - sf0 + 1;
+    if (tid < n_own) {
+      const int kb = sf0 + tid;
+      const int f = (kb <= qb0 ? 1 : 0) | ((second && kb >= sf1) ? 2 : 0);
+      mlist[total + tid] = (uint16_t)(kb | ENT_ORIG | (f << 14));
+    }
+    if (tid == 0) misc[0] = total + n_own;
     __syncthreads();
   }
   const int n_tiles = misc[0];
-  const int own_first = (qb / a.bps) * a.bps;
 
   const uint16_t* pk = a.pk + (int64_t)bh * a.nb * BS * D;
   const uint16_t* pvt = a.pvt + (int64_t)bh * a.nb * BS * D;
-  const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS;
+  const int kvh = h / (a.Hq / a.Hkv);
+  const uint16_t* korig = a.k + b * a.k_sb + kvh * a.k_sh;
+  const uint16_t* ovt = a.ovt + (int64_t)(b * a.Hkv + kvh) * a.nb * BS * D;
 
   // per-lane LDS byte offsets of the fragments inside buffer 0; XOR 0x8000 switches buffer.
   //   K fragment (sub-tile ks, d-step t)      : koff[t] + ks * 8192
@@ -294,7 +330,19 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
 #pragma unroll
   for (int c = 0; c < 8; ++c) voff[c] = LDS_V0 + (uint32_t)(j * 256 + (((2 * c + gh) ^ (j & 15)) * 16));
   const uint32_t lane_off = async_lane_offset(wave, lane);
+  const int qrel8 = 32 * wq + j - 8 * gh;   // query-in-block minus the lane half's key offset
   const float c_log2 = a.scale_log2;
+  // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf` (0 or 0x8000)
+  auto stage_entry = [&](uint32_t e, uint32_t buf) {
+    const int kb_e = (int)(e & ENT_KB);
+    if (e & ENT_ORIG) {
+      stage_krows_async(korig + (int64_t)kb_e * BS * a.k_ss, a.k_ss, a.S - kb_e * BS, buf, wave, lane);
+      stage_tile_async(ovt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+    } else {
+      stage_tile_async(pk + (int64_t)kb_e * BS * D, buf, wave, lane_off);
+      stage_tile_async(pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+    }
+  };
   const uint32_t use_bit = 1u << (14 + grp);
 
   for (int attempt = 0; attempt < 2; ++attempt) {
@@ -308,28 +356,17 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
 
     __syncthreads();   // list build / previous attempt are done with the tile buffers
-    if (n_tiles > 0) {
-      const int kb0 = mlist[0] & 0x3fff;
-      stage_tile_async(pk + (int64_t)kb0 * BS * D, 0, wave, lane_off);
-      stage_tile_async(pvt + (int64_t)kb0 * BS * D, LDS_V0, wave, lane_off);
-      stage_kpos_async(idx + (int64_t)kb0 * BS, LDS_KPOS, wave, lane);
-    }
+    stage_entry((uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[0]), 0u);   // the list is never empty
     for (int it = 0; it < n_tiles; ++it) {
       const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it]);
-      const int kb = ent & 0x3fff;
+      const int kb = (int)(ent & ENT_KB);
       const bool has_next = it + 1 < n_tiles;
-      const int kb_next = has_next ? (__builtin_amdgcn_readfirstlane((int)mlist[it + 1]) & 0x3fff) : 0;
       const uint32_t bufx = (it & 1) ? 0x8000u : 0u;
       __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` has landed
       __syncthreads();                      // every share has; every wave is done with tile it - 1
-      if (has_next) {
-        stage_tile_async(pk + (int64_t)kb_next * BS * D, bufx ^ 0x8000u, wave, lane_off);
-        stage_tile_async(pvt + (int64_t)kb_next * BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
-        stage_kpos_async(idx + (int64_t)kb_next * BS, LDS_KPOS + ((it & 1) ? 0u : 512u), wave, lane);
-      }
+      if (has_next) stage_entry((uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it + 1]), bufx ^ 0x8000u);
       if (!(ent & use_bit) || !qb_valid) continue;
-      const bool masked = kb >= own_first;
-      const uint32_t kpos_lds = LDS_KPOS + ((it & 1) ? 512u : 0u);
+      const bool masked = (ent & ENT_ORIG) && kb == qb;   // the diagonal block; other own-segment blocks lie before it
 
       // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
       // single key yet (its reference maximum is still -inf)
@@ -346,7 +383,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         mx = fmaxf(mx, xhalf_f32(mx));
         m_ref = mx * c_log2;
         all_seen = true;
-        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
+        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
       } else if (first || careful_only || (masked && !all_seen)) {
         // ---------------- careful tile
         first = false;
@@ -358,19 +395,16 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
           for (int t = 0; t < 8; ++t) s[ks] = PBS_MFMA(ldsf((koff[t] ^ bufx) + ks * 8192), qf[t], s[ks]);
         }
         if (masked) {
+          int qrel = 32 * wq + j;
+          asm volatile("" : "+v"(qrel));   // keep the compares inside the tile (see fast_tile)
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks) {
-            __builtin_amdgcn_sched_barrier(0);   // keep the index loads of one sub-tile at a time in flight
+          for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-              const int p = kb * BS + 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1);
-              const int4 ki = *reinterpret_cast<const int4*>(idx + p);
-              if (ki.x > qpos) s[ks][4 * a4 + 0] = -INFINITY;
-              if (ki.y > qpos) s[ks][4 * a4 + 1] = -INFINITY;
-              if (ki.z > qpos) s[ks][4 * a4 + 2] = -INFINITY;
-              if (ki.w > qpos) s[ks][4 * a4 + 3] = -INFINITY;
+            for (int r = 0; r < 16; ++r) {
+              const int a4 = r >> 2;
+              const int key = 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1) + (r & 3);
+              if (key > qrel) s[ks][r] = -INFINITY;
             }
-          }
         }
         float mx = -INFINITY;
 #pragma unroll
@@ -410,8 +444,8 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
             for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff[2 * ks + u] ^ bufx) + dt * 8192), pf, o[dt]);
           }
       } else {
-        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
-        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qpos, kpos_lds, gh);
+        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
+        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
       }
     }
     if (poisoned) misc[1] = 1;
@@ -452,24 +486,29 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
 
 }  // namespace
 
-extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const int32_t* key_indices,
-                                   const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int S,
-                                   int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh,
-                                   int64_t q_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale,
-                                   void* stream) {
-  PBS_REQUIRE(q && perm_k && perm_vt && key_indices && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
+extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k,
+                                   const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B,
+                                   int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size, int64_t q_sb,
+                                   int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb,
+                                   int64_t o_sh, int64_t o_ss, float softmax_scale, void* stream) {
+  PBS_REQUIRE(q && perm_k && perm_vt && k && orig_vt && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_sparse_attn_fwd: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
-  PBS_REQUIRE(B > 0 && Hq > 0 && S > 0, "pbs_sparse_attn_fwd: empty shape");
+  PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_sparse_attn_fwd: bad shape");
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_sparse_attn_fwd: segment_size must be a multiple of block_size");
-  PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && o_sb % 8 == 0 && o_sh % 8 == 0 && o_ss % 8 == 0,
+  PBS_REQUIRE(segment_size / block_size <= 256, "pbs_sparse_attn_fwd: more than 256 blocks per segment");
+  PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && o_sb % 8 == 0 && o_sh % 8 == 0 && o_ss % 8 == 0 &&
+                  k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0,
               "pbs_sparse_attn_fwd: strides must keep rows 16-byte aligned");
-  PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)perm_k % 16) == 0 && ((uintptr_t)perm_vt % 16) == 0,
+  PBS_REQUIRE(k_ss >= D && k_ss < (1 << 22), "pbs_sparse_attn_fwd: key row stride %lld outside [128, 2^22)", (long long)k_ss);
+  PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)perm_k % 16) == 0 &&
+                  ((uintptr_t)perm_vt % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)orig_vt % 16) == 0,
               "pbs_sparse_attn_fwd: pointers must be 16-byte aligned");
   AttnArgs a;
   a.q = (const uint16_t*)q; a.pk = (const uint16_t*)perm_k; a.pvt = (const uint16_t*)perm_vt;
-  a.idx = key_indices; a.cols = csr_cols; a.cnt = csr_cnt; a.o = (uint16_t*)out;
-  a.BH = B * Hq; a.Hq = Hq; a.S = S; a.nb = (S + BS - 1) / BS; a.bps = segment_size / block_size;
-  a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
+  a.k = (const uint16_t*)k; a.ovt = (const uint16_t*)orig_vt;
+  a.cols = csr_cols; a.cnt = csr_cnt; a.o = (uint16_t*)out;
+  a.BH = B * Hq; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS; a.bps = segment_size / block_size;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = (uint32_t)k_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
   a.scale_log2 = softmax_scale * 1.4426950408889634f;
   PBS_REQUIRE(a.nb <= 4096, "pbs_sparse_attn_fwd: more than 4096 blocks per sequence (%d)", a.nb);
   const int heads_per_xcd = (a.BH + 7) / 8;

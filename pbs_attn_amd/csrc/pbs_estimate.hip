@@ -8,6 +8,7 @@
 // waves split the key-block tiles, first to find each row's (max, sum), then to
 // recompute the logits and write P with 128-byte row segments per store.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
 

@@ -4,6 +4,7 @@
 // its power limit), so the benchmark reports it next to the attention kernel's rate as the MFMA ceiling
 // for data like the attention kernel's.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
 

@@ -9,6 +9,7 @@
 // Logits reproduce the rounding points of a bf16 matmul followed by a bf16
 // divide: fp32 accumulate -> bf16 -> / sqrt(D) -> bf16.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
 

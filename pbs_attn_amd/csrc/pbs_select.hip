@@ -10,6 +10,7 @@
 //     kernel has to visit (own-segment blocks whose every key lies after the last
 //     query of the row are dropped from the list: they are fully masked).
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <float.h>
 
 namespace {
@@ -52,7 +53,6 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
   extern __shared__ uint64_t keys[];
   uint8_t* flag = reinterpret_cast<uint8_t*>(keys + a.n_pow2);
   __shared__ int s_first;
-  __shared__ int s_min[256];
   __shared__ int s_scan[256];
   const int qb = blockIdx.x, row = blockIdx.y;
   const int nb = a.nb;
@@ -61,7 +61,6 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
   const int64_t row_off = ((int64_t)row * nb + qb) * nb;
 
   for (int kb = threadIdx.x; kb < nb; kb += blockDim.x) flag[kb] = 0;
-  s_min[threadIdx.x] = INT_MAX;
 
   if (a.thr_is_int_one) {
     __syncthreads();
@@ -121,21 +120,10 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
     const int fb = a.first_blk[row];
     if (fb >= 0 && fb < nb) flag[fb] = 1;
   }
-  // smallest original key position of each own-segment block: one wave per block, shuffle reduction
-  {
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    for (int o = seg_first + wave; o < seg_end; o += (int)(blockDim.x >> 6)) {
-      const int32_t* src = a.idx + (int64_t)row * nb * a.bs + (int64_t)o * a.bs;
-      int v = INT_MAX;
-      for (int i = lane; i < a.bs; i += 64) v = min(v, src[i]);
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) v = min(v, __shfl_xor(v, off, 64));
-      if (lane == 0) s_min[o - seg_first] = v;
-    }
-  }
   __syncthreads();
 
-  const int q_last = min(qb * a.bs + a.bs - 1, a.S - 1);
+  // visit list: the selected blocks of strictly earlier segments (the attention kernel adds the query
+  // block's own segment itself)
   const int per = (nb + 255) / 256;
   const int k0 = threadIdx.x * per, k1 = min(k0 + per, nb);
   int cnt = 0;
@@ -144,8 +132,7 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
     const uint8_t s = flag[kb];
     if (a.sel_mask) a.sel_mask[row_off + kb] = s;
     if (a.final_mask) a.final_mask[row_off + kb] = s | (own ? 1 : 0);
-    const bool visit = own ? (s_min[kb - seg_first] <= q_last) : (s && kb < seg_first);
-    cnt += visit ? 1 : 0;
+    cnt += (s && kb < seg_first) ? 1 : 0;
   }
   s_scan[threadIdx.x] = cnt;
   __syncthreads();
@@ -159,9 +146,7 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
   int w = s_scan[threadIdx.x] - cnt;
   if (a.csr_cols) {
     for (int kb = k0; kb < k1; ++kb) {
-      const bool own = kb >= seg_first && kb < seg_end;
-      const bool visit = own ? (s_min[kb - seg_first] <= q_last) : (flag[kb] && kb < seg_first);
-      if (visit) a.csr_cols[row_off + w++] = kb;
+      if (flag[kb] && kb < seg_first) a.csr_cols[row_off + w++] = kb;
     }
   }
   if (threadIdx.x == 255) a.csr_cnt[(int64_t)row * nb + qb] = s_scan[255];
@@ -236,7 +221,6 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
   const int nb = a.nb;
   const int nb_pad = (nb + 15) & ~15;
   uint8_t* flag = smem_w + wave * nb_pad;
-  int* s_min = reinterpret_cast<int*>(smem_w + 4 * nb_pad) + wave * 256;
   const int64_t rq = (int64_t)blockIdx.x * 4 + wave;   // (row, qb) flattened
   if (rq >= total_rows) return;
   const int row = (int)(rq / nb), qb = (int)(rq % nb);
@@ -332,19 +316,10 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
     const int fb = a.first_blk[row];
     if (fb >= 0 && fb < nb) flag[fb] = 1;
   }
-  for (int o = seg_first; o < seg_end; ++o) {
-    const int32_t* src = a.idx + (int64_t)row * nb * a.bs + (int64_t)o * a.bs;
-    int mv = INT_MAX;
-    for (int i = lane; i < a.bs; i += 64) mv = min(mv, src[i]);
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) mv = min(mv, __shfl_xor(mv, off, 64));
-    if (lane == 0) s_min[o - seg_first] = mv;
-  }
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-  const int q_last = min(qb * a.bs + a.bs - 1, a.S - 1);
   int base = 0;
   for (int kb0 = 0; kb0 < nb; kb0 += 64) {
     const int kb = kb0 + lane;
@@ -354,7 +329,7 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
       const uint8_t sf = flag[kb];
       if (a.sel_mask) a.sel_mask[row_off + kb] = sf;
       if (a.final_mask) a.final_mask[row_off + kb] = sf | (own ? 1 : 0);
-      visit = own ? (s_min[kb - seg_first] <= q_last) : (sf && kb < seg_first);
+      visit = sf && kb < seg_first;   // own-segment blocks are the attention kernel's business
     }
     const uint64_t ballot = __ballot(visit);
     if (visit && a.csr_cols) a.csr_cols[row_off + base + __popcll(ballot & ((1ull << lane) - 1ull))] = kb;
@@ -395,7 +370,7 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   if (nb <= 1024) {
     // one wave per row, four rows per workgroup
     const int total = rows * nb;
-    const size_t lds_w = (size_t)4 * ((nb + 15) & ~15) + 4 * 256 * sizeof(int);
+    const size_t lds_w = (size_t)4 * ((nb + 15) & ~15);
     const dim3 grid((unsigned)((total + 3) / 4));
     if (nb <= 64) hipLaunchKernelGGL(select_blocks_wave_kernel<1>, grid, dim3(256), lds_w, st, a, total);
     else if (nb <= 256) hipLaunchKernelGGL(select_blocks_wave_kernel<4>, grid, dim3(256), lds_w, st, a, total);

@@ -5,6 +5,7 @@
 // equal scores keep ascending index order whatever the network does.  The
 // trailing partial segment and the padding up to a whole block keep identity order.
 #include "pbs_common.h"
+#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
 

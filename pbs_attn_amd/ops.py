@@ -66,8 +66,9 @@ def segment_argsort(scores, seq_len, segment_size, block_size=BLOCK):
     return idx
 
 
-def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean"):
-    """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128), pooled_k (B, Hq, nb, D)."""
+def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False):
+    """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128), pooled_k (B, Hq, nb, D) and, with
+    ``want_orig_vt``, orig_vt (B, Hkv, nb, D, 128): the V blocks in original order, transposed."""
     _check_bf16_cuda(k, v)
     if key_pool_mode not in ("mean", "max"):
         raise ValueError(f"Invalid key_pool_mode: {key_pool_mode}")
@@ -80,10 +81,13 @@ def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean"):
     perm_k = torch.empty((B, Hq, nb * BLOCK, D), dtype=k.dtype, device=k.device)
     perm_vt = torch.empty((B, Hq, nb, D, BLOCK), dtype=k.dtype, device=k.device)
     pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device)
-    _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k),
+    orig_vt = torch.empty((B, Hkv, nb, D, BLOCK), dtype=k.dtype, device=k.device) if want_orig_vt else None
+    _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k), _ptr(orig_vt),
                                  B, Hq, Hkv, S, D, BLOCK, k.stride(0), k.stride(1), k.stride(2),
                                  v.stride(0), v.stride(1), v.stride(2), int(key_pool_mode == "max"), _stream()),
                "pbs_gather_kv")
+    if want_orig_vt:
+        return perm_k, perm_vt, pooled_k, orig_vt
     return perm_k, perm_vt, pooled_k
 
 
@@ -143,20 +147,28 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     return sel, fin, cols, cnt
 
 
-def sparse_attn_fwd(q, perm_k, perm_vt, idx, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
-    _check_bf16_cuda(q, perm_k, perm_vt)
+def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
+    """Attention of every query block over the permuted tiles listed in the CSR (earlier segments) and
+    over the causal part of its own segment, read from the original ``k`` (B, Hkv or Hq, S, D) and
+    ``orig_vt``."""
+    _check_bf16_cuda(q, perm_k, perm_vt, k, orig_vt)
     lib = _lib.load()
-    q = _rows16(q)
+    q, k = _rows16(q), _rows16(k)
     B, Hq, S, D = q.shape
+    Hkv = k.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(D)
     if out is None:
         out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
-    assert perm_k.is_contiguous() and perm_vt.is_contiguous() and idx.is_contiguous()
+    nb = (S + BLOCK - 1) // BLOCK
+    assert perm_k.is_contiguous() and perm_vt.is_contiguous() and orig_vt.is_contiguous()
+    assert perm_k.shape == (B, Hq, nb * BLOCK, D) and perm_vt.shape == (B, Hq, nb, D, BLOCK)
+    assert k.shape == (B, Hkv, S, D) and orig_vt.shape == (B, Hkv, nb, D, BLOCK)
     assert csr_cols.is_contiguous() and csr_cnt.is_contiguous()
-    _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(idx), _ptr(csr_cols), _ptr(csr_cnt),
-                                       _ptr(out), B, Hq, S, D, BLOCK, segment_size,
-                                       q.stride(0), q.stride(1), q.stride(2),
+    assert csr_cols.shape == (B, Hq, nb, nb) and csr_cnt.shape == (B, Hq, nb)
+    _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols),
+                                       _ptr(csr_cnt), _ptr(out), B, Hq, Hkv, S, D, BLOCK, segment_size,
+                                       q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
                                        out.stride(0), out.stride(1), out.stride(2), softmax_scale, _stream()),
                "pbs_sparse_attn_fwd")
     return out

@@ -45,6 +45,13 @@ class PermutedKV:
     perm_vt: torch.Tensor       # (B, Hq, nb, D, 128): V blocks transposed [d][key]
     pooled_k: torch.Tensor      # (B, Hq, nb, D)
     seq_len: int
+    key_states: torch.Tensor = None   # the caller's K (B, Hkv or Hq, S, D), read in place for own-segment tiles
+    orig_vt: torch.Tensor = None      # (B, Hkv, nb, D, 128): V blocks in original order, transposed
+
+    def attention(self, query_states, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
+        """Sparse attention over this permutation (see ops.sparse_attn_fwd)."""
+        return ops.sparse_attn_fwd(query_states, self.perm_k, self.perm_vt, self.key_states, self.orig_vt,
+                                   csr_cols, csr_cnt, segment_size, softmax_scale, out)
 
     def permuted_keys(self):
         return self.perm_k[:, :, :self.seq_len]
@@ -75,9 +82,10 @@ def apply_permutation(query_states, key_states, value_states, block_size, segmen
             _mark("score")
         idx = ops.segment_argsort(scores, S, segment_size, block_size)
         _mark("sort")
-    perm_k, perm_vt, pooled_k = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode)
+    perm_k, perm_vt, pooled_k, orig_vt = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode,
+                                                       want_orig_vt=True)
     _mark("gather")
-    return PermutedKV(idx, perm_k, perm_vt, pooled_k, S)
+    return PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, orig_vt)
 
 
 def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment_size, threshold=0.9, causal=True,
@@ -85,7 +93,8 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
                              want_masks=True, block_attn_scores: Optional[torch.Tensor] = None):
     """Selection phase (pbs.py:29-130 + :209).  Returns a dict with
     block_attn_scores, block_mask (selected | first token), final_mask
-    (| own segment), csr_cols, csr_cnt."""
+    (| own segment), csr_cols / csr_cnt (the selected blocks of strictly earlier
+    segments, ascending: the permuted tiles the attention kernel visits)."""
     assert causal
     assert segment_size % block_size == 0, "segment_size must be a multiple of block_size"
     if query_pool_mode not in ("mean", "max"):
@@ -148,8 +157,7 @@ def permuted_block_sparse_attn_fwd(
     perm = apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode)
     sel = permuted_block_selection(query_states, perm, block_size, segment_size, threshold, causal,
                                    force_select_first_block, query_pool_mode, key_pool_mode, want_masks=False)
-    out = ops.sparse_attn_fwd(query_states, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"],
-                              sel["csr_cnt"], segment_size, 1.0 / math.sqrt(head_dim))
+    out = perm.attention(query_states, sel["csr_cols"], sel["csr_cnt"], segment_size, 1.0 / math.sqrt(head_dim))
     _mark("sparse_attn")
     # queries are not permuted (pbs.py:191-193): un-permutation is the identity
     out = ops.unpermute(out)

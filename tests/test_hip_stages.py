@@ -149,18 +149,15 @@ def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
     sel, fin, cols, cnt = ops.select_blocks(Pm.to(dev), thr_dev, idx_pad.to(dev), S, 128, seg, force_first)
     assert torch.equal(sel.cpu(), ref_sel)
     assert torch.equal(fin.cpu(), ref_fin)
-    # the visit list = final mask restricted to segments not after the query block's,
-    # minus own-segment blocks whose every key lies after the block's last query
+    # the visit list = selected (or first-token) blocks of strictly earlier segments, ascending; the query
+    # block's own segment is added by the attention kernel itself
     cols, cnt = cols.cpu(), cnt.cpu()
     qseg = torch.arange(nb) // bps
-    kmin = idx_pad.view(B, H, nb, 128).min(-1).values
     qbs = range(nb) if nb <= 128 else list(range(0, nb, 37)) + [nb - 1]
     for b in range(B):
         for h in range(H):
             for qb in qbs:
-                q_last = min(qb * 128 + 127, S - 1)
-                want = [kb for kb in range(nb) if ref_fin[b, h, qb, kb] and qseg[kb] <= qseg[qb]
-                        and not (qseg[kb] == qseg[qb] and kmin[b, h, kb] > q_last)]
+                want = [kb for kb in range(nb) if ref_sel[b, h, qb, kb] and qseg[kb] < qseg[qb]]
                 assert cols[b, h, qb, :cnt[b, h, qb]].tolist() == want
 
 
@@ -185,10 +182,11 @@ def _run_attention_case(dev, B, Hq, Hkv, S, seg, thr, seed):
     nb = (S + 127) // 128
     idx_pad = torch.cat([idx, torch.arange(S, nb * 128).expand(B, Hq, -1)], -1).int().contiguous().to(dev)
     # same indices and same block probabilities as the oracle -> same masks (asserted), then attention
-    perm_k, perm_vt, _ = ops.gather_kv(k.to(dev), v.to(dev), idx_pad, Hq)
+    kd, vd = k.to(dev), v.to(dev)
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx_pad, Hq, want_orig_vt=True)
     sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), thr, idx_pad, S, 128, seg, True)
     assert torch.equal(fin.cpu(), mid["final_mask"])
-    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, idx_pad, cols, cnt, seg).cpu()
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, orig_vt, cols, cnt, seg).cpu()
     dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], idx, mid["final_mask"], 128)
     assert_attn_close(out, out_ref, what="HIP vs oracle naive path")
     assert_attn_close(out, dense, what="HIP vs dense fp32 oracle")
@@ -208,7 +206,7 @@ def test_sparse_attention_strided_query(dev):
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     perm = P.apply_permutation(qd, kd, vd, 128, 256)
     sel = P.permuted_block_selection(qd, perm, 128, 256, 0.9)
-    args = (perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], 256)
+    args = (perm.perm_k, perm.perm_vt, perm.key_states, perm.orig_vt, sel["csr_cols"], sel["csr_cnt"], 256)
     q_strided = qd.transpose(1, 2).contiguous().transpose(1, 2)
     assert not q_strided.is_contiguous()
     out_c = ops.sparse_attn_fwd(qd, *args)
@@ -228,7 +226,7 @@ def _pipeline_vs_dense(dev, q, k, v, seg, thr, **kw):
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     perm = P.apply_permutation(qd, kd, vd, 128, seg)
     sel = P.permuted_block_selection(qd, perm, 128, seg, thr, **kw)
-    out = ops.sparse_attn_fwd(qd, perm.perm_k, perm.perm_vt, perm.key_indices, sel["csr_cols"], sel["csr_cnt"], seg)
+    out = perm.attention(qd, sel["csr_cols"], sel["csr_cnt"], seg)
     idx = perm.key_indices.cpu()[:, :, :S].long()
     # permutation stays inside segments
     sc = (S // seg) * seg
