@@ -31,7 +31,7 @@ PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 FLOP_PER_BLOCK_PAIR = 4.0 * 128 * 128 * 128
 # HBM bytes per launch of the attention kernel (fetched + written past L2), from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE scaled by a 1 GiB copy (profiles/pipeline_cfg2_hbm_traffic.txt); only known for that workload.
-MEASURED_ATTN_TRAFFIC_BYTES = {("cfg2", None, 1024, 0.9): 18.78e9 + 1.07e9}
+MEASURED_ATTN_TRAFFIC_BYTES = {("cfg2", None, 1024, 0.9): 20.37e9 + 1.07e9}
 
 
 def log(*a):

@@ -144,13 +144,15 @@ __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
 // exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2); S and P are
 // double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  The MASKED tile
 // (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
-// query: key-in-tile > query-in-block, an arithmetic test (`qrel8` = query-in-block - 8 * lane half).
+// query: key-in-tile > query-in-block, an arithmetic test.
 template <bool MASKED, int PF>
 __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t (&koff)[8],
                                           const uint32_t (&voff)[8], uint32_t bufx, float c_log2, float& m_ref,
-                                          float& l_part, bool& poisoned, int qrel8) {
-  // opaque per call: the 128 mask compares of a diagonal tile depend only on the lane, and hoisted out of
-  // the tile loop they would each pin a 64-bit scalar mask
+                                          float& l_part, bool& poisoned, int wq, int j, int gh) {
+  // query-in-block minus the lane half's key offset; made opaque per call: the 128 mask compares of a
+  // diagonal tile depend only on the lane, and hoisted out of the tile loop they would each pin a 64-bit
+  // scalar mask
+  int qrel8 = 32 * wq + j - 8 * gh;
   if (MASKED) asm volatile("" : "+v"(qrel8));
   const float negm = -m_ref;
   float rsum[4] = {0.f, 0.f, 0.f, 0.f};
@@ -330,7 +332,6 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
 #pragma unroll
   for (int c = 0; c < 8; ++c) voff[c] = LDS_V0 + (uint32_t)(j * 256 + (((2 * c + gh) ^ (j & 15)) * 16));
   const uint32_t lane_off = async_lane_offset(wave, lane);
-  const int qrel8 = 32 * wq + j - 8 * gh;   // query-in-block minus the lane half's key offset
   const float c_log2 = a.scale_log2;
   // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf` (0 or 0x8000)
   auto stage_entry = [&](uint32_t e, uint32_t buf) {
@@ -383,7 +384,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         mx = fmaxf(mx, xhalf_f32(mx));
         m_ref = mx * c_log2;
         all_seen = true;
-        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
+        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
       } else if (first || careful_only || (masked && !all_seen)) {
         // ---------------- careful tile
         first = false;
@@ -444,8 +445,8 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
             for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff[2 * ks + u] ^ bufx) + dt * 8192), pf, o[dt]);
           }
       } else {
-        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
-        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, qrel8);
+        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
+        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
       }
     }
     if (poisoned) misc[1] = 1;
@@ -469,12 +470,17 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     __syncthreads();
     if (qb_valid) {
       uint16_t* obase = a.o + b * a.o_sb + h * a.o_sh;
-      const int t256 = tid & 255;
+      // the query block index is rebuilt from the thread id here: keeping it alive across the tile loop
+      // costs a register the loop does not have
+      int tid_e = threadIdx.x;
+      asm volatile("" : "+v"(tid_e));
+      const int qb_e = 2 * pair + (tid_e >> 8);
+      const int t256 = tid_e & 255;
 #pragma unroll
       for (int n = 0; n < 8; ++n) {
         const int ci = t256 + 256 * n;
         const int row = ci >> 4, c = ci & 15;
-        const int pos = qb * BS + row;
+        const int pos = qb_e * BS + row;
         if (pos < a.S)
           *reinterpret_cast<u32x4*>(obase + (int64_t)pos * a.o_ss + c * 8) =
               *reinterpret_cast<const u32x4*>(os + row * D + ((c ^ (row & 15)) * 8));
