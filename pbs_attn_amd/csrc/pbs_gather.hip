@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
       if (!orig) kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
       vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
     }
-    if (!orig) *reinterpret_cast<u32x4*>(kdst + i * D + c * 8) = kv;
+    if (!orig) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float lo = bf16_bits_to_f32(kv[e] & 0xffffu), hi = bf16_bits_to_f32(kv[e] >> 16);
@@ -97,7 +97,7 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
       const uint32_t lo = vt[(c * 8 + 2 * e) * VT_PITCH + d], hi = vt[(c * 8 + 2 * e + 1) * VT_PITCH + d];
       o[e] = lo | (hi << 16);
     }
-    *reinterpret_cast<u32x4*>(vdst + d * BS + c * 8) = o;
+    __builtin_nontemporal_store(o, reinterpret_cast<u32x4*>(vdst + d * BS + c * 8));
   }
 }
 
