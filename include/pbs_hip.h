@@ -123,6 +123,15 @@ int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out,
                          int key_pool_max, float softmax_scale, void* workspace, size_t workspace_bytes,
                          void* stream);
 
+/* Rotary position embedding of Q and K in one pass: out = bf16(bf16(x * cos) + bf16(rotate_half(x) * sin)),
+ * bit-identical to the bf16 tensor expression of pbs_attn/patch/huggingface.py:14-25 (called at :203).
+ * q (B, Hq, S, 128) and k (B, Hkv, S, 128) with their strides (e.g. the (B, S, H, D) memory of the
+ * projections); cos / sin (B or 1, S, 128) with batch stride c_sb (0 to broadcast) and row stride c_ss;
+ * q_out (B, Hq, S, 128) and k_out (B, Hkv, S, 128) contiguous, head-major. */
+int pbs_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Hq,
+                int Hkv, int S, int head_dim, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh,
+                int64_t k_ss, int64_t c_sb, int64_t c_ss, void* stream);
+
 /* Measurement aid with no counterpart in the reference: `iters` x 8 v_mfma_f32_32x32x16_bf16 per wave on
  * 256 workgroups of 8 waves, operands taken from `operands` (65536 bf16 values of the caller's choice: the
  * sustained rate depends on the values).  `sink` takes 256 * 512 floats, `clocks` (two 64-bit counters the

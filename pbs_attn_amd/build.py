@@ -12,7 +12,7 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpbs_hip.so")
 
 SOURCES = ["pbs_abi.hip", "pbs_score.hip", "pbs_sort.hip", "pbs_gather.hip", "pbs_estimate.hip",
-           "pbs_select.hip", "pbs_attn.hip", "pbs_pipeline.hip", "pbs_probe.hip"]
+           "pbs_select.hip", "pbs_attn.hip", "pbs_pipeline.hip", "pbs_probe.hip", "pbs_rope.hip"]
 
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

@@ -207,6 +207,26 @@ def prefill_attn_fwd(q, k, v, block_size, segment_size, threshold, force_select_
     return out
 
 
+def rope_qk(q, k, cos, sin):
+    """Rotary embedding of q (B, Hq, S, D) and k (B, Hkv, S, D) with cos / sin (B or 1, S, D): the bits of
+    ``x * cos + rotate_half(x) * sin`` in bf16 (pbs_attn/patch/huggingface.py:14-25), in one pass, returned
+    contiguous and head-major."""
+    _check_bf16_cuda(q, k, cos, sin)
+    lib = _lib.load()
+    q, k, cos, sin = _rows16(q), _rows16(k), _rows16(cos), _rows16(sin)
+    B, Hq, S, D = q.shape
+    Hkv = k.shape[1]
+    assert k.shape == (B, Hkv, S, D) and cos.shape == sin.shape and cos.shape[-2:] == (S, D)
+    assert cos.dim() == 3 and cos.shape[0] in (1, B) and cos.stride() == sin.stride()
+    q_out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
+    k_out = torch.empty((B, Hkv, S, D), dtype=q.dtype, device=q.device)
+    c_sb = cos.stride(0) if cos.shape[0] == B and B > 1 else 0
+    _lib.check(lib.pbs_rope_qk(_ptr(q), _ptr(k), _ptr(cos), _ptr(sin), _ptr(q_out), _ptr(k_out), B, Hq, Hkv, S, D,
+                               q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                               c_sb, cos.stride(1), _stream()), "pbs_rope_qk")
+    return q_out, k_out
+
+
 def unpermute(o_perm, q_idx=None, out=None):
     """out[b, h, q_idx[b, h, i]] = o_perm[b, h, i]; identity (no launch) when the
     queries were not permuted."""

@@ -8,9 +8,11 @@ Same surface as the reference's pbs_attn/patch/huggingface.py:
 projections -> RoPE -> KV-cache update -> prefill_fn -> o_proj; single-token
 decode steps go to the module's original forward.
 
-One extension: a prefill function whose underlying python function carries
+Two extensions: a prefill function whose underlying python function carries
 ``native_gqa = True`` receives K/V at the KV-head count, which saves the
-``repeat_kv`` copies (the PBS HIP path reads KV head h // group itself).
+``repeat_kv`` copies (the PBS HIP path reads KV head h // group itself); and bf16
+head-dim-128 prompts on the GPU get their rotary embedding from one HIP kernel
+that produces the same bits as the tensor expression.
 """
 from __future__ import annotations
 
@@ -76,6 +78,13 @@ def _split_heads(x, bsz, q_len, head_dim):
     return x.view(bsz, q_len, n_local, head_dim).transpose(1, 2), n_local
 
 
+def _fused_rope_applies(q, k, cos, sin):
+    return (q.is_cuda and q.dtype == torch.bfloat16 and k.dtype == q.dtype and cos.dtype == q.dtype
+            and sin.dtype == q.dtype and q.shape[-1] == 128 and cos.dim() == 3 and cos.shape == sin.shape
+            and cos.shape[0] in (1, q.shape[0]) and tuple(cos.shape[-2:]) == (q.shape[2], 128)
+            and cos.stride() == sin.stride())
+
+
 def patched_attention_forward(
     self,
     hidden_states: torch.Tensor,
@@ -98,7 +107,12 @@ def patched_attention_forward(
     v, _ = _split_heads(self.v_proj(hidden_states), bsz, q_len, self.head_dim)
 
     cos, sin = position_embeddings
-    q, k = apply_rotary_pos_emb(q, k, cos, sin)
+    if _fused_rope_applies(q, k, cos, sin):
+        # same bits as apply_rotary_pos_emb, one kernel instead of ten, head-major contiguous outputs
+        from pbs_attn_amd import ops
+        q, k = ops.rope_qk(q, k, cos, sin)
+    else:
+        q, k = apply_rotary_pos_emb(q, k, cos, sin)
     if past_key_values is not None:
         past_key_values.update(k, v, self.layer_idx, {"sin": sin, "cos": cos, "cache_position": cache_position})
 

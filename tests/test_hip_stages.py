@@ -376,3 +376,19 @@ def test_single_call_entry_point_rejects_small_workspace(dev):
                                   *st, 0.9, None, 0, 1, 0, 0, 128 ** -0.5, ws.data_ptr(), need - 256,
                                   torch.cuda.current_stream().cuda_stream)
     assert rc < 0 and b"workspace too small" in lib.pbs_last_error()
+
+
+# ---------------------------------------------------------------- rotary embedding of the glue
+@pytest.mark.parametrize("B,Hq,Hkv,S,cos_batch", [(1, 4, 2, 1000, 1), (2, 3, 1, 257, 2), (2, 2, 2, 64, 1)])
+def test_rope_qk_bitwise_equals_the_tensor_expression(dev, B, Hq, Hkv, S, cos_batch):
+    from pbs_attn_amd.patch.huggingface import apply_rotary_pos_emb
+    g = torch.Generator().manual_seed(S)
+    # q, k as the patched forward sees them: transposed views of (B, S, H, D) projections
+    q = (torch.randn((B, S, Hq, 128), generator=g) * 3).bfloat16().to(dev).transpose(1, 2)
+    k = (torch.randn((B, S, Hkv, 128), generator=g) * 3).bfloat16().to(dev).transpose(1, 2)
+    ang = torch.rand((cos_batch, S, 128), generator=g) * 6.28
+    cos, sin = ang.cos().bfloat16().to(dev), ang.sin().bfloat16().to(dev)
+    q_ref, k_ref = apply_rotary_pos_emb(q, k, cos, sin)
+    q_out, k_out = ops.rope_qk(q, k, cos, sin)
+    assert q_out.is_contiguous() and k_out.is_contiguous()
+    assert torch.equal(q_out, q_ref) and torch.equal(k_out, k_ref)
