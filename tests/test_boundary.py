@@ -36,6 +36,35 @@ def test_library_exports_every_declared_symbol():
     assert _lib.load().pbs_abi_version() == 1
 
 
+def test_ctypes_signatures_match_the_header_parameter_by_parameter():
+    # a wrong ctypes signature passes garbage to a kernel launch: compare every declaration's return
+    # type and parameter types with the table the host code calls through
+    from pbs_attn_amd import _lib
+    text = re.sub(r"/\*.*?\*/", "", open(HEADER).read(), flags=re.S)
+    decls = re.findall(r"\b(int|size_t|double|const char\s*\*)\s+(pbs_\w+)\s*\(([^;]*?)\)\s*;", text, flags=re.S)
+    assert len(decls) == len(_lib.SIGNATURES)
+
+    def ctype_of(param):
+        param = " ".join(param.split())
+        if param == "void":
+            return None
+        if "*" in param:
+            return ctypes.c_void_p
+        base = param.rsplit(" ", 1)[0].replace("const ", "")
+        return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "float": ctypes.c_float, "size_t": ctypes.c_size_t,
+                "double": ctypes.c_double}[base]
+
+    ret_map = {"int": ctypes.c_int, "size_t": ctypes.c_size_t, "double": ctypes.c_double}
+    for ret, name, params in decls:
+        want_args = [t for t in (ctype_of(x) for x in params.split(",")) if t is not None]
+        res, args = _lib.SIGNATURES[name]
+        assert list(args) == want_args, f"{name}: ctypes argument types differ from the header"
+        if "char" in ret:
+            assert res is ctypes.c_char_p
+        else:
+            assert res is ret_map[ret], f"{name}: return type differs from the header"
+
+
 def test_argument_errors_are_reported_without_a_gpu():
     from pbs_attn_amd import _lib
     lib = _lib.load()

@@ -392,3 +392,17 @@ def test_rope_qk_bitwise_equals_the_tensor_expression(dev, B, Hq, Hkv, S, cos_ba
     q_out, k_out = ops.rope_qk(q, k, cos, sin)
     assert q_out.is_contiguous() and k_out.is_contiguous()
     assert torch.equal(q_out, q_ref) and torch.equal(k_out, k_ref)
+
+
+def test_mfma_probe_runs_and_counts_clocks(dev):
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    pool = torch.randn(65536, device=dev).bfloat16()
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    rc = lib.pbs_mfma_probe(pool.data_ptr(), 100, sink.data_ptr(), clocks.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    torch.cuda.synchronize()
+    c = clocks.tolist()
+    assert c[0] > 0 and c[1] > 0 and torch.isfinite(sink).all()
+    assert lib.pbs_mfma_probe_flop(100) == 256 * 8 * 100 * 8 * 2.0 * 32 * 32 * 16
