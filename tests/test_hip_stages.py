@@ -406,3 +406,23 @@ def test_mfma_probe_runs_and_counts_clocks(dev):
     c = clocks.tolist()
     assert c[0] > 0 and c[1] > 0 and torch.isfinite(sink).all()
     assert lib.pbs_mfma_probe_flop(100) == 256 * 8 * 100 * 8 * 2.0 * 32 * 32 * 16
+
+
+def test_strided_key_value_views_give_the_same_bits(dev):
+    # K / V handed over as transposed views of (B, S, H, D) projections (what a glue without the fused
+    # rotary kernel produces): every stage reads them in place, the result equals the contiguous run
+    q, k, v = small_case(2, 4, 2, 1111, seed=21)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    ks = kd.transpose(1, 2).contiguous().transpose(1, 2)
+    vs = vd.transpose(1, 2).contiguous().transpose(1, 2)
+    assert not ks.is_contiguous() and not vs.is_contiguous()
+    for thr in (0.9, 1):
+        ref = P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, 256, thr, True)
+        out = P.permuted_block_sparse_attn_fwd(qd, ks, vs, 128, 256, thr, True)
+        assert torch.equal(out, ref)
+        P.stage_timer = _NullTimer()
+        try:
+            staged = P.permuted_block_sparse_attn_fwd(qd, ks, vs, 128, 256, thr, True)
+        finally:
+            P.stage_timer = None
+        assert torch.equal(staged, ref)
