@@ -1,0 +1,91 @@
+"""Seeded sweep over randomly drawn configurations (shapes, head grouping, segment sizes, thresholds,
+pooling modes, ragged lengths): for each one the GPU stages are checked against the CPU oracle --
+indices and masks bit-exactly on the GPU's own score tensors, attention against dense fp32 attention on
+the GPU's own mask -- and the single-call entry point against the staged path."""
+import random
+
+import pytest
+import torch
+
+from oracle import pbs_oracle as O
+from pbs_attn_amd import pbs as P
+from tests.util import assert_attn_close, expand_kv, small_case
+
+pytestmark = pytest.mark.gpu
+
+
+def _draw(seed):
+    r = random.Random(seed)
+    hkv = r.choice([1, 2, 3])
+    hq = hkv * r.choice([1, 2, 4, 7])
+    seg = 128 * r.choice([1, 2, 2, 3, 4, 8])
+    nseg = r.randint(1, 7)
+    tail = r.choice([0, 0, 1, 37, 127, 128, 129, seg - 1])
+    S = max(130, nseg * seg + tail)
+    if S > 3000:
+        S = 3000 - r.randint(0, 200)
+    thr = r.choice([0.5, 0.8, 0.9, 0.95, 0.999, 1.0, 1, "rows"])
+    return dict(B=r.choice([1, 1, 2]), Hq=hq, Hkv=hkv, S=S, seg=seg, thr=thr, force=r.random() < 0.7,
+                qpool=r.choice(["mean", "mean", "max"]), kpool=r.choice(["mean", "mean", "max"]),
+                kind=r.choice(["uniform_heavy", "span_heavy", "local_window", "strong_heavy"]))
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_configuration(dev, seed):
+    c = _draw(seed)
+    B, Hq, Hkv, S, seg = c["B"], c["Hq"], c["Hkv"], c["S"], c["seg"]
+    q, k, v = small_case(B, Hq, Hkv, S, kind=c["kind"], seed=1000 + seed)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    thr = c["thr"]
+    if thr == "rows":
+        thr = (torch.rand((B, Hq), generator=torch.Generator().manual_seed(seed)) * 0.5 + 0.45).to(dev)
+    nb, bps = (S + 127) // 128, seg // 128
+
+    perm = P.apply_permutation(qd, kd, vd, 128, seg, c["kpool"])
+    sel = P.permuted_block_selection(qd, perm, 128, seg, thr, True, c["force"], c["qpool"], c["kpool"])
+    out = perm.attention(qd, sel["csr_cols"], sel["csr_cnt"], seg)
+
+    # permutation: bit-exact with the oracle's stable sort of the GPU's own scores; K / V gathered bitwise
+    idx = perm.key_indices.cpu()[:, :, :S].long()
+    sc = (S // seg) * seg
+    if sc >= 2 * seg or (sc == seg and S > seg):
+        from pbs_attn_amd import ops
+        scores = ops.score_keys(qd, kd, 128, seg).cpu()
+        assert torch.equal(idx, O.segment_argsort(scores, S, seg)), c
+    else:
+        assert torch.equal(idx, torch.arange(S).expand(B, Hq, -1)), c
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    assert torch.equal(perm.permuted_keys().cpu(), O.gather_rows(ke, idx)), c
+    assert torch.equal(perm.permuted_values().cpu(), O.gather_rows(ve, idx)), c
+    # original-order transposed V (zero past S)
+    ovt = perm.orig_vt.cpu().transpose(-1, -2).reshape(B, Hkv, nb * 128, 128)
+    assert torch.equal(ovt[:, :, :S], v) and (ovt[:, :, S:] == 0).all(), c
+
+    # selection: bit-exact with the oracle on the GPU's own block probabilities
+    idx_pad = torch.cat([idx, torch.arange(S, nb * 128).expand(B, Hq, -1)], -1)
+    Pm = sel["block_attn_scores"]
+    is_one = isinstance(thr, int) and thr == 1
+    cand, segm = O.candidate_masks(nb, bps)
+    if is_one:
+        ref_sel = cand.view(1, 1, nb, nb).expand(B, Hq, nb, nb).clone()
+    else:
+        ref_sel = O.select_blocks(Pm.cpu(), thr.cpu() if isinstance(thr, torch.Tensor) else thr)
+    if c["force"]:
+        ref_sel = ref_sel | O.first_token_mask(idx_pad, 128)
+    assert torch.equal(sel["block_mask"].cpu(), ref_sel), c
+    assert torch.equal(sel["final_mask"].cpu(), ref_sel | segm[None, None]), c
+    cnt = sel["csr_cnt"].cpu()
+    assert torch.equal(cnt, (ref_sel & cand[None, None]).sum(-1).int()), c
+
+    # attention: dense fp32 masked attention on the GPU's own indices and mask
+    dense = O.dense_masked_attention_fp32(q, perm.permuted_keys().cpu(), perm.permuted_values().cpu(), idx,
+                                          sel["final_mask"].cpu(), 128)
+    assert_attn_close(out.cpu(), dense, what=f"{c}")
+
+    # the single-call entry point runs the same kernels on the same data
+    one = P.permuted_block_sparse_attn_fwd(qd, kd, vd, 128, seg, thr, True, c["force"], True, c["qpool"], c["kpool"])
+    if S > seg:
+        assert torch.equal(one, out), c
+    else:
+        assert_attn_close(one.cpu(), torch.nn.functional.scaled_dot_product_attention(
+            q.float(), ke.float(), ve.float(), is_causal=True), what=f"S <= segment {c}")
