@@ -38,7 +38,7 @@ constexpr int D = 128;
 constexpr int BS = 128;
 constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
 constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
-constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096 + 257)
+constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096 + 1)
 constexpr uint32_t LDS_MISC = LDS_LIST + 10240;   // ints: [0] merged count, [1] redo flag, [16..24) wave totals
 constexpr uint32_t LDS_TOTAL = LDS_MISC + 1024;   // 142 336 bytes of the CU's 160 KB
 constexpr uint32_t ENT_KB = 0x1fffu;              // visit-list entry: key block ...
@@ -501,7 +501,7 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_sparse_attn_fwd: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
   PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_sparse_attn_fwd: bad shape");
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_sparse_attn_fwd: segment_size must be a multiple of block_size");
-  PBS_REQUIRE(segment_size / block_size <= 256, "pbs_sparse_attn_fwd: more than 256 blocks per segment");
+  PBS_REQUIRE(segment_size / block_size <= 511, "pbs_sparse_attn_fwd: more than 511 blocks per segment");
   PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && o_sb % 8 == 0 && o_sh % 8 == 0 && o_ss % 8 == 0 &&
                   k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0,
               "pbs_sparse_attn_fwd: strides must keep rows 16-byte aligned");

@@ -354,7 +354,6 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_select_blocks: segment_size must be a multiple of block_size");
   const int nb = (S + block_size - 1) / block_size;
   const int bps = segment_size / block_size;
-  PBS_REQUIRE(bps <= 256, "pbs_select_blocks: more than 256 blocks per segment");
   PBS_REQUIRE(nb <= 4096, "pbs_select_blocks: more than 4096 blocks per sequence (%d)", nb);
   PBS_REQUIRE(workspace && workspace_bytes >= pbs_select_blocks_workspace_bytes(rows), "pbs_select_blocks: workspace too small");
   SelectArgs a;

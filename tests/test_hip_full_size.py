@@ -184,3 +184,11 @@ def test_more_than_1024_blocks_per_sequence(dev):
             & (idx[:, :, None, :] <= pos[rows].view(1, 1, -1, 1))
         ref = torch.softmax(logits.masked_fill(~allowed, float("-inf")), -1) @ pv
         assert_attn_close(out[:, :, rows], ref, what=f"q block {qb} of 1300")
+
+
+def test_sequence_inside_one_large_segment_is_plain_causal_attention(dev):
+    # S <= segment_size: the reference calls dense SDPA; here one segment spans the sequence (313 blocks)
+    S = 40000
+    q, k, v = make_qkv(1, 2, 1, S, 128, "uniform_heavy", seed=13, device=dev)
+    out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 65536, 0.9, True)
+    assert_attn_close(out, _sdpa(q, k, v), what="S <= segment_size vs SDPA")
