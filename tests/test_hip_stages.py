@@ -426,3 +426,26 @@ def test_strided_key_value_views_give_the_same_bits(dev):
         finally:
             P.stage_timer = None
         assert torch.equal(staged, ref)
+
+
+def test_single_call_path_can_be_captured_in_a_graph(dev):
+    # nothing on the path allocates, synchronises or clears memory through the runtime: the whole pass can be
+    # recorded once and replayed; every replay (with eager work in between) equals the eager result
+    from pbs_attn_amd.synth import make_qkv
+    q, k, v = make_qkv(1, 8, 2, 2048 + 77, 128, "uniform_heavy", seed=3, device=dev)
+    eager = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 256, 0.9, True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        P.permuted_block_sparse_attn_fwd(q, k, v, 128, 256, 0.9, True)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 256, 0.9, True)
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
+        (q.float() @ q.float().transpose(-1, -2)[..., :64]).sum().item()   # eager work between replays
