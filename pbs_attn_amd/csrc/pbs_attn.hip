@@ -56,6 +56,7 @@ struct AttnArgs {
   uint16_t* o;
   int BH, Hq, Hkv, S, nb, bps;
   uint32_t k_ss;   // key row stride in elements (< 2^22)
+  int xcd_start[9];   // work items (head-major, long rows first) of XCD x: [xcd_start[x], xcd_start[x + 1])
   int64_t q_sb, q_sh, q_ss, k_sb, k_sh, o_sb, o_sh, o_ss;
   float scale_log2;
 };
@@ -218,14 +219,18 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   const int j = lane & 31, gh = lane >> 5;
   const int grp = wave >> 2, wq = wave & 3;
 
-  // workgroup -> (head, pair of query blocks): a head stays on one XCD (blockIdx % 8) and an XCD works
-  // through one head at a time, long rows first, so the workgroups resident on an XCD walk the same
-  // permuted K/V stream at about the same pace and share its tiles in that XCD's L2
+  // workgroup -> (head, pair of query blocks).  The work items, ordered head by head with the long rows of
+  // a head first, are cut into eight contiguous ranges of about equal work, one per XCD (blockIdx % 8):
+  // an XCD works through one head at a time, so its resident workgroups walk the same permuted K/V
+  // stream at about the same pace and share its tiles in that XCD's L2; with fewer heads than XCDs, or
+  // a head count that is no multiple of 8, a head is split between XCDs instead of leaving some idle
   const int npair = (a.nb + 1) >> 1;
   const int w_id = blockIdx.x;
   const int xcd = w_id & 7, slot_id = w_id >> 3;
-  const int bh = (slot_id / npair) * 8 + xcd;
-  const int pair = npair - 1 - slot_id % npair;
+  const int item = a.xcd_start[xcd] + slot_id;
+  if (item >= a.xcd_start[xcd + 1]) return;
+  const int bh = item / npair;
+  const int pair = npair - 1 - item % npair;
   if (bh >= a.BH) return;
   const int b = bh / a.Hq, h = bh % a.Hq;
   const int qb = 2 * pair + grp;
@@ -517,9 +522,29 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = (uint32_t)k_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
   a.scale_log2 = softmax_scale * 1.4426950408889634f;
   PBS_REQUIRE(a.nb <= 4096, "pbs_sparse_attn_fwd: more than 4096 blocks per sequence (%d)", a.nb);
-  const int heads_per_xcd = (a.BH + 7) / 8;
-  const int64_t n_wg = (int64_t)8 * heads_per_xcd * ((a.nb + 1) / 2);
-  PBS_REQUIRE(n_wg < (1ll << 31), "pbs_sparse_attn_fwd: launch too large");
+  // eight ranges of equal estimated work: the row pair p of a head costs about p + 1 (causal length)
+  const int64_t npair = (a.nb + 1) / 2;
+  PBS_REQUIRE((int64_t)a.BH * npair < (1ll << 28), "pbs_sparse_attn_fwd: launch too large");
+  const double head_work = 0.5 * (double)npair * (double)(npair + 1);
+  int max_items = 0;
+  for (int x = 0; x <= 8; ++x) {
+    const double target = head_work * a.BH * x / 8.0;
+    int64_t head = (int64_t)(target / head_work);
+    if (head > a.BH) head = a.BH;
+    const double rem = target - head * head_work;
+    // items of a head in launch order are pairs npair - 1, npair - 2, ...: the first i of them cost
+    // i * npair - i (i - 1) / 2
+    int64_t lo = 0, hi = npair;
+    while (lo < hi) {
+      const int64_t mid = (lo + hi) / 2;
+      if ((double)mid * npair - 0.5 * (double)mid * (mid - 1) >= rem - 1e-6) hi = mid; else lo = mid + 1;
+    }
+    int64_t start = head * npair + (head < a.BH ? lo : 0);
+    if (x == 8) start = (int64_t)a.BH * npair;
+    a.xcd_start[x] = (int)start;
+    if (x > 0) max_items = std::max(max_items, a.xcd_start[x] - a.xcd_start[x - 1]);
+  }
+  const int64_t n_wg = (int64_t)8 * max_items;
   hipError_t attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
   if (attr != hipSuccess) {
     pbs_set_error("pbs_sparse_attn_fwd: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
