@@ -192,3 +192,25 @@ def test_sequence_inside_one_large_segment_is_plain_causal_attention(dev):
     q, k, v = make_qkv(1, 2, 1, S, 128, "uniform_heavy", seed=13, device=dev)
     out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 65536, 0.9, True)
     assert_attn_close(out, _sdpa(q, k, v), what="S <= segment_size vs SDPA")
+
+
+def test_longest_supported_sequence(dev):
+    # 4096 blocks (524 283 tokens, ragged): the limits of the visit list, the long-row selection kernel and
+    # the split of two heads over eight XCDs; sampled rows against dense fp32 attention on the path's own mask
+    S, seg = 4096 * 128 - 5, 1024
+    q, k, v = make_qkv(1, 2, 1, S, 128, "span_heavy", seed=4, device=dev)
+    perm = P.apply_permutation(q, k, v, 128, seg)
+    sel = P.permuted_block_selection(q, perm, 128, seg, 0.9)
+    out = perm.attention(q, sel["csr_cols"], sel["csr_cnt"], seg)
+    assert torch.isfinite(out.float()).all()
+    idx = perm.key_indices[:, :, :S].long()
+    pk, pv = perm.permuted_keys().float(), perm.permuted_values().float()
+    pos = torch.arange(S, device=dev)
+    for qb in (3, 2048, 4095):
+        rows = slice(qb * 128, min(qb * 128 + 128, S))
+        logits = q[:, :, rows].float() @ pk.transpose(-1, -2) / 128 ** 0.5
+        allowed = sel["final_mask"][:, :, qb][:, :, None, :].repeat_interleave(128, -1)[..., :S] \
+            & (idx[:, :, None, :] <= pos[rows].view(1, 1, -1, 1))
+        ref = torch.softmax(logits.masked_fill(~allowed, float("-inf")), -1) @ pv
+        assert_attn_close(out[:, :, rows], ref, what=f"q block {qb} of 4096")
+    assert torch.equal(P.permuted_block_sparse_attn_fwd(q, k, v, 128, seg, 0.9, True), out)
