@@ -50,5 +50,22 @@ def build_library(verbose: bool = False) -> str:
     return LIB_PATH
 
 
+C_SMOKE_SRC = os.path.join(os.path.dirname(HERE), "tests", "c_abi", "smoke.c")
+C_SMOKE_BIN = os.path.join(os.path.dirname(HERE), "tests", "c_abi", "smoke")
+
+
+def build_c_smoke() -> str:
+    """Compiles tests/c_abi/smoke.c with gcc as plain C99 against include/pbs_hip.h and links it to the
+    library and the HIP runtime: the check that the C ABI is usable without Python or torch."""
+    rocm = os.environ.get("ROCM_PATH", "/opt/rocm")
+    cmd = ["gcc", "-std=c99", "-O2", C_SMOKE_SRC, "-I" + os.path.join(os.path.dirname(HERE), "include"),
+           "-I" + os.path.join(rocm, "include"), "-D__HIP_PLATFORM_AMD__", "-o", C_SMOKE_BIN, "-L" + LIB_DIR, "-lpbs_hip",
+           "-L" + os.path.join(rocm, "lib"), "-lamdhip64", "-lm", "-Wl,-rpath,$ORIGIN/../../pbs_attn_amd/lib",
+           "-Wl,-rpath," + os.path.join(rocm, "lib")]
+    subprocess.run(cmd, check=True)
+    return C_SMOKE_BIN
+
+
 if __name__ == "__main__":
     print(build_library(verbose=True))
+    print(build_c_smoke())

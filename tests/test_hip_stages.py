@@ -449,3 +449,15 @@ def test_single_call_path_can_be_captured_in_a_graph(dev):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
         (q.float() @ q.float().transpose(-1, -2)[..., :64]).sum().item()   # eager work between replays
+
+
+def test_library_from_plain_c_without_python_or_torch(dev):
+    # tests/c_abi/smoke.c, built by pbs_attn_amd.build.build_c_smoke (gcc, C99): hipMalloc'ed buffers, one
+    # pbs_prefill_attn_fwd pass, checked on the host against causal attention
+    import os
+    import subprocess
+    from pbs_attn_amd.build import C_SMOKE_BIN
+    assert os.path.exists(C_SMOKE_BIN), "tests/c_abi/smoke is not built: run python -m pbs_attn_amd.build"
+    run = subprocess.run([C_SMOKE_BIN], capture_output=True, text=True, timeout=100)
+    assert run.returncode == 0, run.stdout + run.stderr
+    assert "c_abi_smoke ok" in run.stdout
