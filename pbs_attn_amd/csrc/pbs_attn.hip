@@ -1,12 +1,19 @@
-// Block-sparse flash-attention forward over permuted keys (bf16, head_dim 128).
+// Block-sparse flash-attention forward of PBS-Attn (bf16, head_dim 128).
 //
+// What a query block attends to
+//   * the permuted K / V tiles of the selected key blocks of EARLIER segments (the visit list), no mask;
+//   * its own segment, read from the ORIGINAL K and the original-order transposed V: blocks
+//     first-of-segment .. query block, with the plain causal triangle on the last one (the diagonal block).
+//     A segment's permuted blocks hold the same keys as its original blocks and attention does not depend
+//     on key order, so this is the reference's "every block of the own segment, element mask original key
+//     position > query position" with half the tiles and one masked tile instead of all.
 // Work decomposition
 //   One workgroup (8 waves, two per SIMD) owns TWO adjacent 128-query blocks of one head.  Waves
 //   0-3 serve the first block, waves 4-7 the second, 32 queries per wave.  The two visit lists
-//   (ascending key-block indices) are merged once into LDS; every merged key block is copied ONCE
-//   into LDS for both query blocks, which halves the L2 -> LDS traffic and doubles the time a tile
-//   stays in flight.  K and V tiles are double-buffered (2 x 64 KB) and fetched one tile ahead with
-//   asynchronous global -> LDS copies (no registers), one workgroup barrier per tile.
+//   (ascending key-block indices) are merged once into LDS, the own-segment blocks appended; every merged
+//   tile is copied ONCE into LDS for both query blocks, which halves the L2 -> LDS traffic and doubles
+//   the time a tile stays in flight.  K and V tiles are double-buffered (2 x 64 KB) and fetched one tile
+//   ahead with asynchronous global -> LDS copies (no registers), one workgroup barrier per tile.
 // Data layout
 //   K tile: 128 keys x 128 d row-major; V tile: stored TRANSPOSED in HBM by the gather kernel,
 //   128 d x 128 keys.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
@@ -19,16 +26,15 @@
 //   Softmax runs in the exp2 domain in fp32; P is rounded to bf16 before P.V and the row sum uses
 //   the unrounded values; the output is normalised once at the end.
 // Tile kinds
-//   * fast tiles (earlier segments, after the first): a software pipeline over the four 32-key
-//     sub-tiles -- S of sub-tile k+1, exponentials of sub-tile k and P.V of sub-tile k-1 are issued
-//     interleaved, LDS fragments are read three slots ahead.  Exponentials are taken against a LAZY
-//     reference maximum: it is not updated per tile; a row sum of one tile above 2^14 triggers a
-//     uniform rescale (exact, all terms share the reference); an overflow marks the row and the
-//     whole workgroup redoes it without speculation.
-//     Tiles of the query block's own segment run the same pipeline with the element mask "original
-//     key position > query position"; the tile's key positions travel to LDS with the tile.
-//   * careful tiles (a row that starts inside its own segment, own-segment tiles while some query has
-//     seen no key yet, and the redo pass): all of S first, exact running maximum, classic online softmax.
+//   * fast tiles: a software pipeline over the four 32-key sub-tiles -- S of sub-tile k+1, exponentials
+//     of sub-tile k and P.V of sub-tile k-1 are issued interleaved, LDS fragments are read three slots
+//     ahead.  Exponentials are taken against a LAZY reference maximum: it is not updated per tile; a row
+//     sum of one tile above 2^14 triggers a uniform rescale (exact, all terms share the reference); an
+//     overflow marks the row and the whole workgroup redoes it without speculation.  The first tile of a
+//     row takes its reference from the exact maximum over its first 32 keys.  The diagonal tile runs the
+//     same pipeline and zeroes the exponentials of keys after the query (key-in-tile > query-in-block).
+//   * careful tiles (a row whose first tile is the diagonal one, and the redo pass): all of S first,
+//     exact running maximum, classic online softmax.
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
