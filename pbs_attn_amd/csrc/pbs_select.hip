@@ -6,9 +6,11 @@
 //     float64, every prefix rounded to float32 and compared with float32(threshold),
 //   * keep ranks <= the first prefix that reaches the threshold (none if never),
 //   * OR in the block holding original key 0 (optional) and the row's own segment,
-//   * emit the dense byte masks and the ascending list of key blocks the attention
-//     kernel has to visit (own-segment blocks whose every key lies after the last
-//     query of the row are dropped from the list: they are fully masked).
+//   * emit the dense byte masks and the visit list: the ascending selected key blocks of
+//     strictly earlier segments (the attention kernel adds the causal part of the row's
+//     own segment itself, in original key order).
+// Rows of up to 1024 blocks take the wave-level variant further down (one wave per row,
+// the row in registers).
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <float.h>
