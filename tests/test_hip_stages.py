@@ -461,3 +461,20 @@ def test_library_from_plain_c_without_python_or_torch(dev):
     run = subprocess.run([C_SMOKE_BIN], capture_output=True, text=True, timeout=100)
     assert run.returncode == 0, run.stdout + run.stderr
     assert "c_abi_smoke ok" in run.stdout
+
+
+@pytest.mark.parametrize("B,H,S", [(1, 2, 300), (2, 3, 1025)])
+def test_unpermute_scatter_and_identity(dev, B, H, S):
+    # out[b, h, q_idx[b, h, i]] = o_perm[b, h, i]; without an index it is the identity and launches nothing
+    g = torch.Generator().manual_seed(S)
+    o_perm = torch.randn((B, H, S, 128), generator=g).bfloat16().to(dev)
+    q_idx = torch.stack([torch.stack([torch.randperm(S, generator=g) for _ in range(H)]) for _ in range(B)]).int().to(dev)
+    out = ops.unpermute(o_perm, q_idx)
+    ref = torch.empty_like(o_perm)
+    ref.scatter_(2, q_idx.long().unsqueeze(-1).expand(-1, -1, -1, 128), o_perm)
+    assert torch.equal(out, ref)
+    # into a strided destination
+    buf = torch.empty((B, S, H, 128), dtype=o_perm.dtype, device=dev).transpose(1, 2)
+    ops.unpermute(o_perm, q_idx, out=buf)
+    assert torch.equal(buf, ref)
+    assert ops.unpermute(o_perm) is o_perm
