@@ -36,6 +36,20 @@ int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, i
                    int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
                    int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream);
 
+/* pbs_score_keys without a workspace argument and without any allocation.  It has no counterpart in
+ * the reference: it is for callers that cannot allocate device memory around the call (code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc).  The chunk partials and row
+ * statistics live in a library-owned device array of PBS_SCORE_KEYS_STATIC_SCRATCH_BYTES per GPU (held
+ * until the process ends); shapes whose pbs_score_keys_workspace_bytes exceeds it are rejected with an
+ * argument error (-1).  The device address of the array is looked up on the first call on each device
+ * (-2 if that fails).  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * two threads) race; calls on one stream are ordered and safe.  Same arguments, results and error
+ * behaviour as pbs_score_keys otherwise. */
+#define PBS_SCORE_KEYS_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
+int pbs_score_keys_static(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
+                          int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
+                          int64_t k_sh, int64_t k_ss, void* stream);
+
 /* Per-segment stable descending argsort (ties keep ascending index).
  * scores: (rows, Sc); key_indices: (rows, S_pad) int32 global key positions;
  * positions >= Sc (trailing partial segment, block padding) keep identity order.

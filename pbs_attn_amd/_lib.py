@@ -15,6 +15,7 @@ SIGNATURES = {
     "pbs_last_error": (c_char_p, []),
     "pbs_score_keys_workspace_bytes": (_Z, [_I, _I, _I, _I, _I]),
     "pbs_score_keys": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _Z, _P]),
+    "pbs_score_keys_static": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "pbs_segment_argsort": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "pbs_gather_kv": (c_int, [_P] * 7 + [_I] * 6 + [_L] * 6 + [_I, _P]),
     "pbs_pool_q": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P]),

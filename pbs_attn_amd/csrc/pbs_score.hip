@@ -10,6 +10,7 @@
 // divide: fp32 accumulate -> bf16 -> / sqrt(D) -> bf16.
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
+#include <mutex>
 
 namespace {
 
@@ -212,22 +213,28 @@ extern "C" size_t pbs_score_keys_workspace_bytes(int B, int Hq, int Hkv, int S, 
   return (size_t)B * Hq * ((size_t)chunks_for(Sc, chunk_keys_for(B, Hq, Hkv, Sc)) + 1) * NQ * 2 * sizeof(float);
 }
 
-extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
-                              int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
-                              int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream) {
-  PBS_REQUIRE(q && k && scores, "pbs_score_keys: null tensor pointer");
-  PBS_REQUIRE(head_dim == D, "pbs_score_keys: head_dim must be 128, got %d", head_dim);
-  PBS_REQUIRE(block_size == NQ, "pbs_score_keys: block_size must be 128, got %d", block_size);
-  PBS_REQUIRE(B > 0 && Hkv > 0 && Hq > 0 && Hq % Hkv == 0, "pbs_score_keys: bad head counts Hq=%d Hkv=%d", Hq, Hkv);
-  PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_score_keys: segment_size %d not a multiple of block_size", segment_size);
-  PBS_REQUIRE(S >= NQ, "pbs_score_keys: sequence shorter than one block");
+namespace {
+
+// Argument checks and the three launches shared by the two entry points; `workspace` holds the chunk
+// partials and the folded row statistics.
+int score_keys_launch(const char* who, const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S,
+                      int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                      int64_t k_sb, int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream) {
+  PBS_REQUIRE(q && k && scores, "%s: null tensor pointer", who);
+  PBS_REQUIRE(head_dim == D, "%s: head_dim must be 128, got %d", who, head_dim);
+  PBS_REQUIRE(block_size == NQ, "%s: block_size must be 128, got %d", who, block_size);
+  PBS_REQUIRE(B > 0 && Hkv > 0 && Hq > 0 && Hq % Hkv == 0, "%s: bad head counts Hq=%d Hkv=%d", who, Hq, Hkv);
+  PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "%s: segment_size %d not a multiple of block_size", who, segment_size);
+  PBS_REQUIRE(S >= NQ, "%s: sequence shorter than one block", who);
   PBS_REQUIRE(q_ss % 8 == 0 && k_ss % 8 == 0 && q_sh % 8 == 0 && k_sh % 8 == 0 && q_sb % 8 == 0 && k_sb % 8 == 0,
-              "pbs_score_keys: strides must keep rows 16-byte aligned");
-  PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0, "pbs_score_keys: pointers must be 16-byte aligned");
+              "%s: strides must keep rows 16-byte aligned", who);
+  PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0, "%s: pointers must be 16-byte aligned", who);
+  PBS_REQUIRE((int64_t)B * Hkv <= 65535, "%s: too many KV heads (%lld)", who, (long long)B * Hkv);
   const int Sc = (S / segment_size) * segment_size;
   if (Sc == 0) return 0;
   PBS_REQUIRE(workspace && workspace_bytes >= pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size),
-              "pbs_score_keys: workspace too small");
+              "%s: workspace too small (%zu < %zu bytes)", who, workspace_bytes,
+              pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size));
   ScoreArgs a;
   a.q = (const uint16_t*)q;
   a.k = (const uint16_t*)k;
@@ -246,5 +253,66 @@ extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B
   hipLaunchKernelGGL(score_kernel<false>, grid, block, 0, st, a);
   hipLaunchKernelGGL(score_reduce_kernel, dim3(B * Hq), dim3(NQ), 0, st, a);
   hipLaunchKernelGGL(score_kernel<true>, grid, block, 0, st, a);
-  return pbs_check_launch("pbs_score_keys");
+  return pbs_check_launch(who);
+}
+
+}  // namespace
+
+extern "C" int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,
+                              int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb,
+                              int64_t k_sh, int64_t k_ss, void* workspace, size_t workspace_bytes, void* stream) {
+  return score_keys_launch("pbs_score_keys", q, k, scores, B, Hq, Hkv, S, head_dim, block_size, segment_size, q_sb, q_sh,
+                           q_ss, k_sb, k_sh, k_ss, workspace, workspace_bytes, stream);
+}
+
+// ---- the variant that allocates nothing: chunk partials and row statistics live in a library-owned
+// device array.  Every GPU holds its own copy of the array at its own address; the address is looked up
+// once per device, on that device's first call, and only that pointer is ever handed to kernels.
+namespace {
+
+constexpr size_t SCRATCH_BYTES = PBS_SCORE_KEYS_STATIC_SCRATCH_BYTES;   // 8 MiB per GPU, held until the process ends
+static __device__ __align__(256) unsigned char scratch[SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_ptr[MAX_DEVICES] = {};
+
+// device pointer of `scratch` on the current device (null + error message on failure)
+void* scratch_on_current_device(const char* who) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    pbs_set_error("%s: cannot identify the current device (%s, device %d)", who, hipGetErrorString(e), dev);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(g_scratch_lock);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !p) {
+      pbs_set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", who, dev, hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  return g_scratch_ptr[dev];
+}
+
+}  // namespace
+
+extern "C" int pbs_score_keys_static(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S,
+                                     int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh,
+                                     int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, void* stream) {
+  PBS_REQUIRE(B > 0 && Hkv > 0 && Hq > 0 && Hq % Hkv == 0 && S > 0 && segment_size > 0,
+              "pbs_score_keys_static: bad shape B=%d Hq=%d Hkv=%d S=%d segment_size=%d", B, Hq, Hkv, S, segment_size);
+  const size_t need = pbs_score_keys_workspace_bytes(B, Hq, Hkv, S, segment_size);
+  PBS_REQUIRE(need <= SCRATCH_BYTES,
+              "pbs_score_keys_static: this shape needs %zu bytes of scratch memory, the library-owned buffer holds %zu; "
+              "use pbs_score_keys with a caller-provided workspace", need, SCRATCH_BYTES);
+  void* ws = scratch_on_current_device("pbs_score_keys_static");
+  if (!ws) return -2;
+  // every partial and statistic the later launches read is written by the earlier ones of this call:
+  // nothing needs clearing between calls
+  return score_keys_launch("pbs_score_keys_static", q, k, scores, B, Hq, Hkv, S, head_dim, block_size, segment_size,
+                           q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, ws, SCRATCH_BYTES, stream);
 }
