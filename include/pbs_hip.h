@@ -84,6 +84,12 @@ int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim
 int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows, int nb,
                              int head_dim, int blocks_per_segment, void* stream);
 
+/* The same with the candidate rule of the reference's un-permuted MeanPooling baseline: query block qb
+ * scores every key block kb <= qb (the causal lower triangle INCLUDING the diagonal), so no row is NaN.
+ * Replaces pbs_attn/baselines/MeanPooling.py:43-48 (mask) + pbs_attn/src/utils.py:30-33. */
+int pbs_block_logits_softmax_causal(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows,
+                                    int nb, int head_dim, void* stream);
+
 /* Cumulative-threshold selection.  threshold_per_row (rows floats) overrides
  * `threshold` when non-null; threshold_is_int_one selects every candidate.
  * sel_mask = selected | first-token block; final_mask = sel_mask | own segment

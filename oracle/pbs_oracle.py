@@ -191,7 +191,8 @@ def select_blocks(block_attn_scores: torch.Tensor, threshold: Union[float, torch
     sorted_scores, sorted_idx = torch.sort(p, dim=-1, descending=True, stable=True)
     cum = torch.cumsum(sorted_scores.double(), dim=-1).float()
     if isinstance(threshold, torch.Tensor):
-        thr = threshold.to(torch.float32).reshape(threshold.shape + (1, 1))
+        # utils.py:70-72: compared after torch's type promotion (a float64 tensor makes it a float64 compare)
+        thr = threshold.reshape(threshold.shape + (1, 1))
     else:
         thr = torch.tensor(float(threshold), dtype=torch.float32)
     exceed = cum >= thr
@@ -321,3 +322,48 @@ def visited_block_pairs(final_mask: torch.Tensor, blocks_per_segment: int) -> in
     qb = torch.arange(nb).unsqueeze(1) // blocks_per_segment
     kb = torch.arange(nb).unsqueeze(0) // blocks_per_segment
     return int((final_mask & (kb <= qb)).sum())
+
+
+# --------------------------------------------------------------------------
+# MeanPooling baseline (no permutation) -- baselines/MeanPooling.py:7-99
+# --------------------------------------------------------------------------
+
+def meanpooling_selection(q, k, block_size, threshold, force_select_first_block=True,
+                          force_select_current_block=True):
+    """baselines/MeanPooling.py:24-58: pad to whole blocks, candidates = the causal lower triangle of blocks
+    INCLUDING the diagonal (:43-46), block_pooled_attn + select_blocks on the un-permuted keys (:48-50),
+    column 0 forced (:52-53), diagonal forced (:54-58).  Returns (block_attn_scores, block_mask)."""
+    k = _expand_to(q, k)
+    b, h, s, _ = q.shape
+    ident = torch.arange(s).view(1, 1, -1).expand(b, h, -1)
+    pq, _ = pad_to_block(q, ident, block_size)
+    pk, _ = pad_to_block(k, ident, block_size)
+    nb = pq.shape[2] // block_size
+    cand = torch.tril(torch.ones(nb, nb, dtype=torch.bool))
+    scores = block_pooled_attn(pq, pk, block_size, cand)
+    block_mask = select_blocks(scores, threshold)
+    if force_select_first_block:
+        block_mask[:, :, :, 0] = True
+    if force_select_current_block:
+        block_mask = block_mask | torch.eye(nb, dtype=torch.bool).view(1, 1, nb, nb)
+    return scores, block_mask
+
+
+def meanpooling_prefill(q, k, v, block_size=128, segment_size=1024, threshold=0.9, causal=True,
+                        force_select_first_block=True, force_select_current_block=True,
+                        return_intermediates=False):
+    """baselines/MeanPooling.py:7-99 with the external block-sparse kernel (:80-96, ``is_causal=True``)
+    restated as what it computes: attention over the selected blocks with the token-level causal mask, here
+    through the same naive per-block path as PBS (identity key order).  ``segment_size`` is accepted and
+    unused, as there."""
+    assert causal
+    k, v = _expand_to(q, k), _expand_to(q, v)
+    assert q.shape[2] == k.shape[2]
+    b, h, s, _ = q.shape
+    scores, block_mask = meanpooling_selection(q, k, block_size, threshold, force_select_first_block,
+                                               force_select_current_block)
+    ident = torch.arange(s).view(1, 1, -1).expand(b, h, -1)
+    out = sparse_attn_naive(q, k, v, ident, block_mask, block_size)
+    if return_intermediates:
+        return out, dict(block_attn_scores=scores, block_mask=block_mask, key_indices=ident)
+    return out

@@ -37,6 +37,7 @@
 //     exact running maximum, classic online softmax.
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
+#include <atomic>
 
 namespace {
 
@@ -82,8 +83,9 @@ __device__ __forceinline__ int mfma_row_to_key(int i) {
 // (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4).  That chunk does not depend on n: one
 // per-lane byte offset serves the four loads, tile base and LDS base advance by 8192 bytes in
 // scalar registers.  The copy is issued from inline assembly so that the compiler does not order
-// later LDS reads of the OTHER buffer behind it; completion is awaited with s_waitcnt vmcnt(0)
-// before the barrier that publishes the tile.
+// later LDS reads of the OTHER buffer behind it; M0 is handed over as a register operand (the compiler
+// writes it and knows it is in use; the s_nop is the wait state between that write and the copy);
+// completion is awaited with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
 __device__ __forceinline__ uint32_t async_lane_offset(int wave, int lane) {
   const int row = 4 * wave + (lane >> 4);
   const int c = (lane & 15) ^ (row & 15);
@@ -100,9 +102,8 @@ __device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t l
 #pragma unroll
   for (int n = 0; n < 4; ++n) {
     const uint64_t base = srcu + n * 8192;
-    const uint32_t m0v = lds0 + n * 8192;
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(lane_off), "s"(base)
-                 : "memory");
+    register uint32_t m0v asm("m0") = lds0 + n * 8192;
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(lane_off), "s"(base) : "memory");
   }
 }
 
@@ -124,18 +125,16 @@ __device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t 
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       const uint64_t base = srcu + (uint64_t)n * (64u * row_stride);
-      const uint32_t m0v = lds0 + n * 8192;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base)
-                   : "memory");
+      register uint32_t m0v asm("m0") = lds0 + n * 8192;
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base) : "memory");
     }
   } else {
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
       const uint32_t row = min(r0 + 32u * n, (uint32_t)(rows_valid - 1));
       const uint32_t voff = row * row_stride * 2u + c16;
-      const uint32_t m0v = lds0 + n * 8192;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu)
-                   : "memory");
+      register uint32_t m0v asm("m0") = lds0 + n * 8192;
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu) : "memory");
     }
   }
 }
@@ -501,6 +500,8 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   }
 }
 
+std::atomic<uint64_t> g_lds_reserved{0};   // bit d: the kernel's LDS size has been raised on device d
+
 }  // namespace
 
 extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k,
@@ -551,7 +552,14 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
     if (x > 0) max_items = std::max(max_items, a.xcd_start[x] - a.xcd_start[x - 1]);
   }
   const int64_t n_wg = (int64_t)8 * max_items;
-  hipError_t attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
+  // the kernel's dynamic LDS size is raised once per device, not per call
+  int dev = 0;
+  hipError_t attr = hipGetDevice(&dev);
+  const bool tracked = attr == hipSuccess && dev >= 0 && dev < 64;
+  if (attr == hipSuccess && !(tracked && (g_lds_reserved.load(std::memory_order_acquire) >> dev & 1))) {
+    attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
+    if (attr == hipSuccess && tracked) g_lds_reserved.fetch_or(1ull << dev, std::memory_order_release);
+  }
   if (attr != hipSuccess) {
     pbs_set_error("pbs_sparse_attn_fwd: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
     return (int)attr;

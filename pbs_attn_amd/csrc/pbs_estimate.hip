@@ -21,6 +21,15 @@ __device__ __forceinline__ float logit_round(float acc, float sqrt_d) {
   return round_bf16(round_bf16(acc) / sqrt_d);
 }
 
+// number of candidate key blocks of query block qb (its candidates are key blocks 0 .. count - 1): the blocks
+// of strictly earlier segments, or -- CAUSAL, the rule of the reference's un-permuted MeanPooling baseline --
+// every block up to and including the diagonal one
+template <bool CAUSAL>
+__device__ __forceinline__ int candidate_count(int qb, int bps) {
+  return CAUSAL ? qb + 1 : (qb / bps) * bps;
+}
+
+template <bool CAUSAL>
 __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_t* pooled_q, const uint16_t* pooled_k,
                                                                    float* P, int nb, int bps, float sqrt_d) {
   __shared__ float s_m[4][32], s_l[4][32];
@@ -33,7 +42,7 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
   float* out = P + (int64_t)bh * nb * nb;
 
   const int q_last = min(32 * qt + 31, nb - 1);
-  const int cand_max = (q_last / bps) * bps;        // candidates of the tile's last row
+  const int cand_max = candidate_count<CAUSAL>(q_last, bps);   // candidates of the tile's last row
   const int n_kt_cand = (cand_max + 31) / 32;
   const int n_kt_all = (nb + 31) / 32;
 
@@ -46,7 +55,7 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
 
   // ---- pass A: per query block (column j) running max / sum over its candidates
   const int qb_col = 32 * qt + j;
-  const int cand_col = qb_col < nb ? (qb_col / bps) * bps : 0;
+  const int cand_col = qb_col < nb ? candidate_count<CAUSAL>(qb_col, bps) : 0;
   float m_run = -INFINITY, l_run = 0.f;
   for (int kt = wave; kt < n_kt_cand; kt += 4) {
     const uint16_t* row = pk + (int64_t)min(32 * kt + j, nb - 1) * D;
@@ -107,7 +116,7 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
       const int ql = 8 * (r >> 2) + 4 * half + (r & 3);
       const int qb = 32 * qt + ql;
       if (qb < nb && kb < nb) {
-        const int cand = (qb / bps) * bps;
+        const int cand = candidate_count<CAUSAL>(qb, bps);
         float p;
         if (cand == 0) p = __uint_as_float(0x7fc00000u);
         else if (kb < cand) p = __expf(logit_round(acc[r], sqrt_d) - s_max[ql]) * s_inv[ql];
@@ -120,13 +129,32 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
 
 }  // namespace
 
+namespace {
+int launch_block_logits(const char* who, bool causal, const void* pooled_q, const void* pooled_k, float* block_attn_scores,
+                        int rows, int nb, int head_dim, int blocks_per_segment, void* stream) {
+  PBS_REQUIRE(pooled_q && pooled_k && block_attn_scores, "%s: null tensor pointer", who);
+  PBS_REQUIRE(head_dim == D, "%s: head_dim must be 128, got %d", who, head_dim);
+  PBS_REQUIRE(rows > 0 && rows <= 65535 && nb > 0 && blocks_per_segment > 0, "%s: bad shape", who);
+  const dim3 grid((nb + 31) / 32, rows);
+  const float sqrt_d = (float)sqrt((double)head_dim);
+  if (causal)
+    hipLaunchKernelGGL(block_logits_softmax_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
+                       (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);
+  else
+    hipLaunchKernelGGL(block_logits_softmax_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
+                       (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);
+  return pbs_check_launch(who);
+}
+}  // namespace
+
 extern "C" int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows,
                                         int nb, int head_dim, int blocks_per_segment, void* stream) {
-  PBS_REQUIRE(pooled_q && pooled_k && block_attn_scores, "pbs_block_logits_softmax: null tensor pointer");
-  PBS_REQUIRE(head_dim == D, "pbs_block_logits_softmax: head_dim must be 128, got %d", head_dim);
-  PBS_REQUIRE(rows > 0 && rows <= 65535 && nb > 0 && blocks_per_segment > 0, "pbs_block_logits_softmax: bad shape");
-  hipLaunchKernelGGL(block_logits_softmax_kernel, dim3((nb + 31) / 32, rows), dim3(256), 0, (hipStream_t)stream,
-                     (const uint16_t*)pooled_q, (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment,
-                     (float)sqrt((double)head_dim));
-  return pbs_check_launch("pbs_block_logits_softmax");
+  return launch_block_logits("pbs_block_logits_softmax", false, pooled_q, pooled_k, block_attn_scores, rows, nb, head_dim,
+                             blocks_per_segment, stream);
+}
+
+extern "C" int pbs_block_logits_softmax_causal(const void* pooled_q, const void* pooled_k, float* block_attn_scores,
+                                               int rows, int nb, int head_dim, void* stream) {
+  return launch_block_logits("pbs_block_logits_softmax_causal", true, pooled_q, pooled_k, block_attn_scores, rows, nb,
+                             head_dim, 1, stream);
 }

@@ -73,6 +73,10 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
     segment_size = (S + block_size - 1) / block_size * block_size;
     threshold_is_int_one = 1;
   }
+  // checked here, before anything is enqueued (the attention kernel holds one segment's blocks in its list)
+  PBS_REQUIRE(segment_size / block_size <= 511,
+              "pbs_prefill_attn_fwd: a segment of %d blocks exceeds the limit of 511 (a sequence that fits inside "
+              "one segment may be at most 65408 tokens; use a smaller segment_size)", segment_size / block_size);
   const Layout L = make_layout(B, Hq, Hkv, S, head_dim, block_size, segment_size);
   PBS_REQUIRE(workspace && workspace_bytes >= L.total, "pbs_prefill_attn_fwd: workspace too small (%zu < %zu bytes)",
               workspace_bytes, L.total);

@@ -51,6 +51,21 @@ __global__ __launch_bounds__(1024) void first_token_block_kernel(const int32_t* 
   if (threadIdx.x == 0) first_blk[blockIdx.x] = found;
 }
 
+__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int lane_mask) {
+  const uint32_t lo = __shfl_xor((uint32_t)v, lane_mask, 64), hi = __shfl_xor((uint32_t)(v >> 32), lane_mask, 64);
+  return ((uint64_t)hi << 32) | lo;
+}
+__device__ __forceinline__ double shfl_up_f64(double v, int delta) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __shfl_up((uint32_t)u, delta, 64), hi = __shfl_up((uint32_t)(u >> 32), delta, 64);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+__device__ __forceinline__ double readlane_f64(double v, int lane) {
+  const uint64_t u = __builtin_bit_cast(uint64_t, v);
+  const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)u, lane), hi = __builtin_amdgcn_readlane((int)(uint32_t)(u >> 32), lane);
+  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
+}
+
 __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
   extern __shared__ uint64_t keys[];
   uint8_t* flag = reinterpret_cast<uint8_t*>(keys + a.n_pow2);
@@ -81,37 +96,69 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
       keys[i] = key;
     }
     bitonic_sort_lds(keys, a.n_pow2);
-    if (threadIdx.x == 0) {
-      // sequential float64 running sum, every prefix rounded to float32 (what torch's CPU cumsum does).
-      // Chunks of 16 sorted values are fetched together and summed without branches, so the serial
-      // chain is 16 double additions; the first qualifying rank is picked from bit masks afterwards.
+    if (threadIdx.x < 64) {
+      // Running sum of the sorted row by ONE wave: lane l owns the `per` consecutive ranks from l * per.  The
+      // sum is first taken as a parallel float64 prefix (local sums + wave scan), which differs from the
+      // sequential float64 sum torch's CPU cumsum forms by < 1e-12; "float32(prefix) >= threshold" is decided
+      // from it unless a prefix up to the first hit lies within 1e-11 of the float32 rounding boundary of the
+      // threshold -- only then the exact sequential sum is evaluated, lane after lane.  Either way the decision
+      // is the sequential sum's.
+      const int lane = threadIdx.x;
+      const int per = a.n_pow2 / 64;   // n_pow2 >= 2048 here
       const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
+      const int r_lo = lane * per;
       double c = 0.0;
-      int first = -1;
-      for (int r0 = 0; r0 < nb; r0 += 16) {
-        float v[16];
-#pragma unroll
-        for (int u = 0; u < 16; ++u) v[u] = desc_key_value(keys[min(r0 + u, a.n_pow2 - 1)]);
-        uint32_t reach = 0, zero = 0;
-#pragma unroll
-        for (int u = 0; u < 16; ++u) {
-          c += (double)v[u];
-          reach |= ((float)c >= thr ? 1u : 0u) << u;
-          zero |= (v[u] == 0.f ? 1u : 0u) << u;
-        }
-        const uint32_t valid = (nb - r0 >= 16) ? 0xffffu : ((1u << (nb - r0)) - 1u);
-        reach &= valid;
-        zero &= valid;
-        // a zero ends the search (sorted: nothing positive follows) unless the threshold is reached
-        // at or before it
-        const int ur = reach ? __builtin_ctz(reach) : 32, uz = zero ? __builtin_ctz(zero) : 32;
-        if (ur <= uz && ur < 32) {
-          first = r0 + ur;
-          break;
-        }
-        if (uz < 32) break;
+      for (int u = 0; u < per; ++u) {
+        const int r = r_lo + u;
+        c += r < nb ? (double)desc_key_value(keys[r]) : 0.0;
       }
-      s_first = first;
+      double incl = c;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const double t = shfl_up_f64(incl, d);
+        if (lane >= d) incl += t;
+      }
+      double excl = shfl_up_f64(incl, 1);
+      if (lane == 0) excl = 0.0;
+      const double mid = 0.5 * ((double)thr + (double)nextafterf(thr, -INFINITY));
+      const double tol = 1e-11 * fmax(1.0, fabs(mid));
+      int my_first = INT_MAX, my_amb = INT_MAX;   // first reaching rank / first ambiguous rank of this lane
+      {
+        double cp = excl;
+        for (int u = 0; u < per; ++u) {
+          const int r = r_lo + u;
+          if (r >= nb) break;
+          cp += (double)desc_key_value(keys[r]);
+          if (my_first == INT_MAX && (float)cp >= thr) my_first = r;
+          if (my_amb == INT_MAX && fabs(cp - mid) <= tol) my_amb = r;
+        }
+      }
+      int first = my_first, amb = my_amb;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        first = min(first, __shfl_xor(first, off, 64));
+        amb = min(amb, __shfl_xor(amb, off, 64));
+      }
+      if (amb <= first && amb != INT_MAX) {
+        // exact sequential sum: lane after lane, each continuing from the lane before
+        double carry = 0.0;
+        first = INT_MAX;
+        for (int L = 0; L < 64 && first == INT_MAX; ++L) {
+          double cs = carry;
+          int hit = INT_MAX;
+          if (lane == L) {
+            for (int u = 0; u < per; ++u) {
+              const int r = r_lo + u;
+              if (r >= nb) break;
+              cs += (double)desc_key_value(keys[r]);
+              if (hit == INT_MAX && (float)cs >= thr) hit = r;
+            }
+          }
+          carry = readlane_f64(cs, L);
+          first = __builtin_amdgcn_readlane(hit, L);
+        }
+      }
+      if (lane == 0) s_first = (first == INT_MAX || first >= nb) ? -1 : first;
     }
     __syncthreads();
     const int first = s_first;
@@ -166,21 +213,6 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
 //     decision is the one the sequential float64 sum gives;
 //   * flags, own-segment minima, masks and the compacted visit list as in the block-level kernel.
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ uint64_t shfl_xor_u64(uint64_t v, int lane_mask) {
-  const uint32_t lo = __shfl_xor((uint32_t)v, lane_mask, 64), hi = __shfl_xor((uint32_t)(v >> 32), lane_mask, 64);
-  return ((uint64_t)hi << 32) | lo;
-}
-__device__ __forceinline__ double shfl_up_f64(double v, int delta) {
-  const uint64_t u = __builtin_bit_cast(uint64_t, v);
-  const uint32_t lo = __shfl_up((uint32_t)u, delta, 64), hi = __shfl_up((uint32_t)(u >> 32), delta, 64);
-  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
-}
-__device__ __forceinline__ double readlane_f64(double v, int lane) {
-  const uint64_t u = __builtin_bit_cast(uint64_t, v);
-  const uint32_t lo = __builtin_amdgcn_readlane((int)(uint32_t)u, lane), hi = __builtin_amdgcn_readlane((int)(uint32_t)(u >> 32), lane);
-  return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
-}
-
 template <int NPL>
 __device__ __forceinline__ void wave_bitonic_sort(uint64_t (&k)[NPL], int lane) {
   constexpr int N = 64 * NPL;

@@ -36,6 +36,27 @@ def _check_bf16_cuda(*ts):
             raise _lib.PbsHipError(f"PBS HIP kernels are bf16 only, got {t.dtype}")
 
 
+def _threshold_args(threshold, B, H, device):
+    """(is_int_one, per-row fp32 tensor or None, python float) with the reference's comparison semantics
+    (pbs_attn/src/pbs.py:120, pbs_attn/src/utils.py:67-72): ``isinstance(threshold, int) and threshold == 1``
+    (True included) selects every candidate; a python float is compared in float32; a tensor is compared
+    after type promotion with the float32 running sum -- for a float64 tensor that is a float64 compare,
+    which equals a float32 compare with the smallest float32 not below the threshold."""
+    if isinstance(threshold, torch.Tensor):
+        t = threshold.to(device=device)
+        if t.dtype == torch.float64:
+            t32 = t.float()
+            t32 = torch.where(t32.double() < t, torch.nextafter(t32, torch.full_like(t32, float("inf"))), t32)
+        elif t.is_floating_point():
+            t32 = t.float()
+        else:
+            t32 = t.double().float()   # integer tensors: exact for every value a threshold can sensibly take
+        return False, t32.expand(B, H).contiguous(), 0.0
+    if isinstance(threshold, int) and threshold == 1:
+        return True, None, 0.0
+    return False, None, float(threshold)
+
+
 def score_keys(q, k, block_size, segment_size):
     """(B, Hq, Sc) float32 key scores; permute_states.py:44-50."""
     _check_bf16_cuda(q, k)
@@ -105,15 +126,21 @@ def pool_q(q, query_pool_mode="mean"):
     return pooled
 
 
-def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment):
-    """(B, H, nb, nb) float32 block probabilities; utils.py:30-33."""
+def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment, causal_candidates=False):
+    """(B, H, nb, nb) float32 block probabilities; utils.py:30-33.  Candidates of a query block are the key
+    blocks of strictly earlier segments (pbs.py:97-107) or, with ``causal_candidates``, every block up to and
+    including the diagonal one (baselines/MeanPooling.py:43-48)."""
     _check_bf16_cuda(pooled_q, pooled_k)
     lib = _lib.load()
     pooled_q, pooled_k = pooled_q.contiguous(), pooled_k.contiguous()
     B, H, nb, D = pooled_q.shape
     P = torch.empty((B, H, nb, nb), dtype=torch.float32, device=pooled_q.device)
-    _lib.check(lib.pbs_block_logits_softmax(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D,
-                                            blocks_per_segment, _stream()), "pbs_block_logits_softmax")
+    if causal_candidates:
+        _lib.check(lib.pbs_block_logits_softmax_causal(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D, _stream()),
+                   "pbs_block_logits_softmax_causal")
+    else:
+        _lib.check(lib.pbs_block_logits_softmax(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D,
+                                                blocks_per_segment, _stream()), "pbs_block_logits_softmax")
     return P
 
 
@@ -125,13 +152,7 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     B, H = idx.shape[:2]
     dev = idx.device
     nb = (seq_len + block_size - 1) // block_size
-    is_int_one = isinstance(threshold, int) and not isinstance(threshold, bool) and threshold == 1
-    thr_rows = None
-    thr = 0.0
-    if isinstance(threshold, torch.Tensor):
-        thr_rows = threshold.to(device=dev, dtype=torch.float32).expand(B, H).contiguous()
-    elif not is_int_one:
-        thr = float(threshold)
+    is_int_one, thr_rows, thr = _threshold_args(threshold, B, H, dev)
     P = None
     if not is_int_one:
         P = block_attn_scores.contiguous()
@@ -188,12 +209,12 @@ def prefill_attn_fwd(q, k, v, block_size, segment_size, threshold, force_select_
     Hkv = k.shape[1]
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(D)
-    is_int_one = isinstance(threshold, int) and not isinstance(threshold, bool) and threshold == 1
-    thr_rows, thr = None, 0.0
-    if isinstance(threshold, torch.Tensor):
-        thr_rows = threshold.to(device=q.device, dtype=torch.float32).expand(B, Hq).contiguous()
-    elif not is_int_one:
-        thr = float(threshold)
+    is_int_one, thr_rows, thr = _threshold_args(threshold, B, Hq, q.device)
+    seg_blocks = (S + block_size - 1) // block_size if S <= segment_size else segment_size // block_size
+    if seg_blocks > 511:
+        raise _lib.PbsHipError(
+            f"a segment of {seg_blocks} blocks exceeds the attention kernel's limit of 511 (a sequence that fits "
+            f"inside one segment may be at most 65408 tokens): use a smaller segment_size")
     out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
     ws_bytes = lib.pbs_prefill_attn_workspace_bytes(B, Hq, Hkv, S, D, block_size, segment_size)
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)

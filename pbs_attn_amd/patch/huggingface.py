@@ -44,7 +44,55 @@ def repeat_kv(hidden_states: torch.Tensor, n_rep: int) -> torch.Tensor:
     return hidden_states.unsqueeze(2).expand(b, h, n_rep, s, d).reshape(b, h * n_rep, s, d)
 
 
-# ---- prefill kernel factory ---------------------------------------------------
+# ---- prefill kernel factories --------------------------------------------------
+
+def get_meanpooling_prefill(block_size=128, segment_size=1024, threshold=0.9,
+                            force_select_first_block=True, force_select_current_block=True):
+    """The un-permuted MeanPooling baseline (pbs_attn/patch/huggingface.py:43-58), through the PBS HIP kernels."""
+    try:
+        from pbs_attn_amd.meanpooling import MeanPooling_prefill as _MeanPooling_prefill
+    except Exception as e:
+        raise RuntimeError("MeanPooling unavailable.") from e
+    return partial(
+        _MeanPooling_prefill,
+        block_size=block_size,
+        segment_size=segment_size,
+        threshold=threshold,
+        causal=True,
+        force_select_first_block=force_select_first_block,
+        force_select_current_block=force_select_current_block,
+    )
+
+
+def _unavailable(name):
+    # the reference builds these baselines on external CUDA packages (minference, block_sparse_attn, flash_attn)
+    # and raises this error when the package is missing (pbs_attn/patch/huggingface.py:60-138); this build
+    # never has them
+    raise RuntimeError(f"{name} unavailable.")
+
+
+def get_minference_prefill(vertical_size=1000, slash_size=6096, adaptive_budget=None):
+    """pbs_attn/patch/huggingface.py:60-88: needs the `minference` CUDA package."""
+    _unavailable("Minference")
+
+
+def get_xattention_prefill(stride, norm=1, threshold=0.8, block_size=128, use_triton=True,
+                           kdb=1, chunk_size=None, keep_sink=False, keep_recent=False):
+    """pbs_attn/patch/huggingface.py:91-110: needs the `block_sparse_attn` CUDA package."""
+    _unavailable("XAttention")
+
+
+def get_flexprefill_prefill(gamma=0.9, tau=0, min_budget=None, max_budget=None,
+                            gqa_interleave=False, softmax_scale=None, block_size=128):
+    """pbs_attn/patch/huggingface.py:112-127: needs the `flash_attn` CUDA package."""
+    _unavailable("FlexPrefill")
+
+
+def get_flashattn_prefill(causal=True):
+    """pbs_attn/patch/huggingface.py:129-138: needs the `flash_attn` CUDA package."""
+    _unavailable("FlashAttn")
+
+
 
 def get_permuted_block_sparse_attn_fwd(
     block_size=128,

@@ -1,10 +1,12 @@
 """PBS-Attn prefill attention on MI355X: host orchestration of the HIP stages.
 
-Mirrors the operator interface of the reference (pbs_attn/src/pbs.py:132-257 and
-:29-130, pbs_attn/src/permute_states.py:87-106): same function names, argument
-meaning, defaults and assertions.  Every stage runs in hand-written gfx950
-kernels reached through the C ABI of libpbs_hip.so; nothing here computes on the
-CPU and nothing falls back to another implementation.
+``permuted_block_sparse_attn_fwd`` mirrors the reference's operator (pbs_attn/src/pbs.py:132-257): same
+name, arguments, defaults and assertions.  ``apply_permutation`` and ``permuted_block_selection`` here are
+this build's own staged API (device-side ``PermutedKV`` bundle, CSR visit list); the functions with the
+reference's signatures and return values are in ``pbs_attn_amd.compat`` and are what
+``pbs_attn.src.pbs`` / ``pbs_attn.src.permute_states`` / ``pbs_attn.src.utils`` export.  Every stage runs
+in hand-written gfx950 kernels reached through the C ABI of libpbs_hip.so; nothing here computes on
+the CPU and nothing falls back to another implementation.
 
 Differences a caller can see:
   * K/V may arrive at the KV-head count (the reference wants them repeated to the
@@ -102,7 +104,7 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
     if key_pool_mode not in ("mean", "max"):
         raise ValueError(f"Invalid key_pool_mode: {key_pool_mode}")
     S = query_states.shape[2]
-    is_int_one = isinstance(threshold, int) and not isinstance(threshold, bool) and threshold == 1
+    is_int_one = isinstance(threshold, int) and threshold == 1   # pbs.py:120 (True counts, as there)
     P = block_attn_scores
     if P is None and (not is_int_one or want_masks):
         pooled_q = ops.pool_q(query_states, query_pool_mode)

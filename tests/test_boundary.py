@@ -84,6 +84,82 @@ def test_reference_import_paths():
     assert a is b and callable(apply_patch_with_prefill) and callable(get_permuted_block_sparse_attn_fwd)
 
 
+def test_reference_callers_import_lines_work():
+    # the import statements of the reference's own callers (eval/efficiency/eval_efficiency.py:21-29,
+    # eval/benchmarks/opencompass_models.py:14-21) and of its stage modules
+    from pbs_attn.patch.huggingface import (  # noqa: F401
+        apply_patch_with_prefill,
+        get_flexprefill_prefill,
+        get_minference_prefill,
+        get_xattention_prefill,
+        get_meanpooling_prefill,
+        get_permuted_block_sparse_attn_fwd,
+        get_flashattn_prefill,
+    )
+    from pbs_attn.src.permute_states import apply_permutation, last_block_attn_sorting
+    from pbs_attn.src.utils import block_pooled_attn, select_blocks
+    from pbs_attn.src.pbs import first_token_mask, permuted_block_selection
+    from pbs_attn.src.pbs import apply_permutation as ap2
+    from pbs_attn.baselines.MeanPooling import MeanPooling_prefill
+    assert ap2 is apply_permutation
+
+    def params(fn):
+        return fn.__code__.co_varnames[:fn.__code__.co_argcount]
+    # the reference's signatures (permute_states.py:6-11,87-93; utils.py:6-13,38-42; pbs.py:10-13,29-41)
+    assert params(last_block_attn_sorting) == ("queries", "keys", "block_size", "segment_size")
+    assert params(apply_permutation) == ("query_states", "key_states", "block_size", "segment_size")
+    assert params(block_pooled_attn) == ("query_states", "key_states", "block_size", "mask", "query_pool_mode",
+                                         "key_pool_mode")
+    assert params(select_blocks) == ("block_attn_scores", "threshold", "causal")
+    assert params(first_token_mask) == ("key_indices", "block_size")
+    assert params(permuted_block_selection) == (
+        "permuted_query_states", "permuted_key_states", "query_indices", "key_indices", "block_size", "segment_size",
+        "threshold", "causal", "force_select_first_block", "query_pool_mode", "key_pool_mode")
+    assert params(MeanPooling_prefill)[:9] == (
+        "query_states", "key_states", "value_states", "block_size", "segment_size", "threshold", "causal",
+        "force_select_first_block", "force_select_current_block")
+    # the baselines built on external CUDA packages fail the way the reference does without them
+    for factory, name in ((get_flashattn_prefill, "FlashAttn"), (get_minference_prefill, "Minference"),
+                          (get_flexprefill_prefill, "FlexPrefill")):
+        with pytest.raises(RuntimeError, match=f"{name} unavailable."):
+            factory()
+    with pytest.raises(RuntimeError, match="XAttention unavailable."):
+        get_xattention_prefill(stride=8)
+    mp = get_meanpooling_prefill()
+    assert isinstance(mp, partial) and mp.func.__name__ == "MeanPooling_prefill"
+    assert mp.keywords == dict(block_size=128, segment_size=1024, threshold=0.9, causal=True,
+                               force_select_first_block=True, force_select_current_block=True)
+    assert "layer_idx" not in mp.func.__code__.co_varnames
+
+
+def test_candidate_rule_detection_of_the_stage_adapter():
+    from pbs_attn_amd.compat import _candidate_rule
+    from oracle import pbs_oracle as O
+    assert _candidate_rule(torch.tril(torch.ones(9, 9, dtype=torch.bool))) == ("causal", 1)
+    for nb, bps in ((8, 2), (12, 4), (7, 1), (9, 9)):
+        assert _candidate_rule(O.candidate_masks(nb, bps)[0]) == ("segments", bps)
+    with pytest.raises(ValueError):
+        _candidate_rule(torch.ones(4, 4, dtype=torch.bool))
+
+
+def test_threshold_argument_semantics():
+    from pbs_attn_amd.ops import _threshold_args
+    dev = torch.device("cpu")
+    assert _threshold_args(1, 1, 2, dev)[0] is True
+    assert _threshold_args(True, 1, 2, dev)[0] is True       # isinstance(True, int): the reference's rule (pbs.py:120)
+    assert _threshold_args(1.0, 1, 2, dev) == (False, None, 1.0)
+    # a float64 tensor is compared in float64 there: the smallest float32 not below it gives the same decisions
+    t64 = torch.tensor([[0.9, 0.5]], dtype=torch.float64)
+    _, rows, _ = _threshold_args(t64, 1, 2, dev)
+    assert rows.dtype == torch.float32 and (rows.double() >= t64).all()
+    assert rows[0, 0].item() == torch.nextafter(torch.tensor(0.9, dtype=torch.float32), torch.tensor(2.0)).item()
+    assert rows[0, 1].item() == 0.5
+    c = torch.tensor([0.9], dtype=torch.float32)            # float32(0.9) < 0.9 in float64
+    assert not bool((c.double() >= t64[0, 0]).item()) and not bool((c >= rows[0, 0]).item())
+    _, rows32, _ = _threshold_args(torch.tensor([[0.9, 0.5]]), 1, 2, dev)
+    assert rows32[0, 0].item() == torch.tensor(0.9, dtype=torch.float32).item()
+
+
 def test_factory_defaults_and_introspection():
     from pbs_attn.patch.huggingface import get_permuted_block_sparse_attn_fwd
     fn = get_permuted_block_sparse_attn_fwd()

@@ -11,7 +11,7 @@ import torch
 import torch.nn.functional as F
 
 from oracle import pbs_oracle as O
-from tests.util import expand_kv, quantised_scores, small_case
+from tests.util import assert_attn_close, expand_kv, quantised_scores, small_case
 
 GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "tiny_pipeline.json")
 
@@ -249,3 +249,67 @@ def test_against_pure_python_vectors():
         assert mid["final_mask"][0, 0].tolist() == exp["final_mask"]
         probs = torch.nan_to_num(mid["block_attn_scores"][0, 0], nan=0.0)
         assert torch.allclose(probs, torch.tensor(exp["block_probs"], dtype=torch.float32), atol=1e-6)
+
+
+# ---------------------------------------------------------------- MeanPooling baseline (no permutation)
+def _brute_meanpooling_mask(q, k, bs, thr, force_first, force_current):
+    """Independent restatement with explicit loops: float64 pooled logits rounded the way the bf16 tensor
+    path rounds them, softmax over kb <= qb, minimal descending prefix (sequential float64 sum rounded to
+    float32 per step), column 0, diagonal."""
+    import numpy as np
+    B, H, S, D = q.shape
+    nb = (S + bs - 1) // bs
+    out = torch.zeros((B, H, nb, nb), dtype=torch.bool)
+    qf = torch.zeros((B, H, nb * bs, D)); qf[:, :, :S] = q.float()
+    kf = torch.zeros((B, H, nb * bs, D)); kf[:, :, :S] = k.float()
+    pq = qf.view(B, H, nb, bs, D).mean(-2).bfloat16()
+    pk = kf.view(B, H, nb, bs, D).mean(-2).bfloat16()
+    for b in range(B):
+        for h in range(H):
+            logit = (pq[b, h] @ pk[b, h].T)                      # bf16 matmul, as the tensor path
+            logit = (logit / math.sqrt(D))                        # bf16 divide
+            for qb in range(nb):
+                row = logit[qb, :qb + 1].float()
+                p = torch.softmax(row, -1).numpy().astype(np.float32)
+                order = sorted(range(qb + 1), key=lambda i: (-p[i], i))
+                c, chosen, reached = np.float64(0.0), [], False
+                for i in order:
+                    c = c + np.float64(p[i])
+                    chosen.append(i)
+                    if np.float32(c) >= np.float32(thr):
+                        reached = True
+                        break
+                if reached:
+                    out[b, h, qb, chosen] = True
+                if force_first:
+                    out[b, h, qb, 0] = True
+                if force_current:
+                    out[b, h, qb, qb] = True
+    return out
+
+
+@pytest.mark.parametrize("S,thr,ff", [(1024, 0.9, True), (900, 0.8, True), (640, 0.95, False)])
+def test_meanpooling_selection_matches_brute_force(S, thr, ff):
+    q, k, _ = small_case(1, 2, 2, S, seed=S)
+    scores, mask = O.meanpooling_selection(q, k, 128, thr, ff, True)
+    assert not torch.isnan(scores).any()                        # the diagonal is a candidate: no empty rows
+    nb = mask.shape[-1]
+    assert torch.allclose(scores.sum(-1), torch.ones(1, 2, nb), atol=1e-5)
+    assert (scores.triu(1) == 0).all()
+    brute = _brute_meanpooling_mask(q, k, 128, thr, ff, True)
+    # rows where two blocks tie exactly on the threshold step are the only place the two may differ
+    assert (mask != brute).float().mean().item() < 2e-2
+    assert (mask.diagonal(dim1=-2, dim2=-1)).all() and not mask.triu(1).any()
+    if ff:
+        assert mask[..., 0].all()
+
+
+def test_meanpooling_prefill_is_dense_attention_on_its_mask():
+    q, k, v = small_case(1, 2, 1, 1000, seed=8)
+    out, mid = O.meanpooling_prefill(q, k, v, 128, 1024, 0.9, return_intermediates=True)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    dense = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128)
+    assert_attn_close(out, dense, max_abs=2.5e-2, what="MeanPooling naive vs dense fp32")
+    # threshold 1.0 on a row whose float32 running sum reaches 1: everything selected -> causal attention
+    full, mid1 = O.meanpooling_prefill(q, k, v, 128, 1024, 0.0, return_intermediates=True)
+    assert mid1["block_mask"].sum() <= mid["block_mask"].sum()  # threshold 0: the top block (+ forced ones) only
