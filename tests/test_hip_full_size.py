@@ -74,9 +74,9 @@ def test_permutation_gather_and_sort_properties_at_32k(dev):
     assert torch.equal(a, b)
 
 
-@pytest.mark.parametrize("thr", [0.8, 0.9, 0.95])
-def test_selection_invariants_at_32k(dev, thr):
-    S, seg, Hq, Hkv = 32768, 256, 8, 2
+@pytest.mark.parametrize("thr,seg", [(0.8, 256), (0.9, 256), (0.95, 256), (0.8, 1024), (0.95, 1024)])
+def test_selection_invariants_at_32k(dev, thr, seg):
+    S, Hq, Hkv = 32768, 8, 2
     nb, bps = S // 128, seg // 128
     q, k, v = make_qkv(1, Hq, Hkv, S, 128, "uniform_heavy", seed=4, device=dev)
     perm = P.apply_permutation(q, k, v, 128, seg)

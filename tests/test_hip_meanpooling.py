@@ -1,0 +1,86 @@
+"""GPU parity of the un-permuted MeanPooling mode (baselines/MeanPooling.py) and of the stage adapters with
+the reference's signatures, against the CPU oracle, through the C ABI."""
+import pytest
+import torch
+
+from oracle import pbs_oracle as O
+from pbs_attn_amd import compat, ops
+from pbs_attn_amd.meanpooling import MeanPooling_prefill
+from tests.util import assert_attn_close, expand_kv, small_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("nb", [8, 33, 100])
+def test_causal_candidate_block_probabilities(dev, nb):
+    g = torch.Generator().manual_seed(nb)
+    pq = (torch.randn((2, 3, nb, 128), generator=g) * 0.5).bfloat16()
+    pk = (torch.randn((2, 3, nb, 128), generator=g) * 0.5).bfloat16()
+    ref = O.block_logits_softmax(pq, pk, torch.tril(torch.ones(nb, nb, dtype=torch.bool)))
+    got = ops.block_logits_softmax(pq.to(dev), pk.to(dev), 1, causal_candidates=True).cpu()
+    assert not torch.isnan(got).any() and (got.triu(1) == 0).all()
+    assert torch.allclose(got.sum(-1), torch.ones(2, 3, nb), atol=1e-4)
+    assert torch.allclose(got, ref, rtol=3e-2, atol=1e-6)
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,thr,ff", [(1, 4, 2, 2048, 0.9, True), (2, 2, 2, 1000, 0.8, True),
+                                               (1, 7, 1, 1536, 0.95, False)])
+def test_meanpooling_masks_bit_exact_and_output_vs_dense(dev, B, Hq, Hkv, S, thr, ff):
+    q, k, v = small_case(B, Hq, Hkv, S, seed=S + Hq)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref_out, mid = O.meanpooling_prefill(q, ke, ve, 128, 1024, thr, True, ff, True, return_intermediates=True)
+    nb = (S + 127) // 128
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    idx = torch.arange(nb * 128, dtype=torch.int32, device=dev).view(1, 1, -1).expand(B, Hq, -1).contiguous()
+    # the selection on the ORACLE's block probabilities: masks must be bit-exact
+    sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, ff)
+    assert torch.equal(fin.cpu(), mid["block_mask"])
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128).cpu()
+    dense = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128)
+    assert_attn_close(out, dense, what="MeanPooling HIP vs dense fp32 on the oracle's mask")
+    assert_attn_close(ref_out, dense, max_abs=2.5e-2, what="oracle naive vs dense fp32")
+    # the whole mode from raw Q, K, V: its own mask differs from the oracle's only where a block probability
+    # sits on the threshold step; its output is dense attention on ITS mask
+    out2, got = MeanPooling_prefill(qd, kd, vd, 128, 1024, thr, True, ff, True, return_masks=True)
+    own_mask = got["block_mask"].cpu()
+    agree = (own_mask == mid["block_mask"]).float().mean().item()
+    assert agree >= 0.995, agree
+    dense2 = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], own_mask, 128)
+    assert_attn_close(out2.cpu(), dense2, what="MeanPooling_prefill vs dense fp32 on its own mask")
+
+
+def test_meanpooling_through_the_factory_and_patch(dev):
+    from pbs_attn.patch.huggingface import get_meanpooling_prefill
+    q, k, v = small_case(1, 4, 4, 1024, seed=3)
+    fn = get_meanpooling_prefill(threshold=0.9)
+    out = fn(q.to(dev), k.to(dev), v.to(dev))
+    assert out.shape == q.shape and torch.isfinite(out.float()).all()
+    with pytest.raises(NotImplementedError):
+        get_meanpooling_prefill(force_select_current_block=False)(q.to(dev), k.to(dev), v.to(dev))
+
+
+def test_stage_adapters_with_the_reference_signatures(dev):
+    B, H, S, seg, thr = 1, 4, 1536, 512, 0.9
+    q, k, v = small_case(B, H, H, S, seed=17)
+    qd, kd = q.to(dev), k.to(dev)
+    perm_k, idx = compat.apply_permutation(qd, kd, 128, seg)
+    assert perm_k.shape == k.shape and idx.shape == (B, H, S) and idx.dtype == torch.int64
+    # a permutation inside every segment, and the gathered rows are the rows of K
+    assert torch.equal(idx.view(B, H, S // seg, seg).sort(-1).values.cpu(),
+                       torch.arange(S).view(1, 1, S // seg, seg).expand(B, H, -1, -1))
+    assert torch.equal(perm_k.cpu(), O.gather_rows(k, idx.cpu()))
+    # selection on these permuted keys: probabilities close to the oracle's, mask bit-exact on the oracle's scores
+    scores, block_mask, segment_mask = compat.permuted_block_selection(qd, perm_k, None, idx, 128, seg, thr)
+    ref_scores, ref_mask, ref_segm = O.permuted_block_selection(q, perm_k.cpu(), idx.cpu(), 128, seg, thr)
+    assert torch.equal(segment_mask.cpu(), ref_segm)
+    nan = torch.isnan(ref_scores)
+    assert torch.equal(torch.isnan(scores.cpu()), nan)
+    assert torch.allclose(scores.cpu()[~nan], ref_scores[~nan], rtol=3e-2, atol=1e-6)
+    assert (block_mask.cpu() == ref_mask).float().mean().item() >= 0.99
+    sel = compat.select_blocks(ref_scores.to(dev), thr)
+    assert torch.equal(sel.cpu(), O.select_blocks(ref_scores, thr))
+    cand, _ = O.candidate_masks(S // 128, seg // 128)
+    P = compat.block_pooled_attn(qd, perm_k, 128, cand.to(dev))
+    assert torch.allclose(P.cpu()[~nan], ref_scores[~nan], rtol=3e-2, atol=1e-6)
+    assert torch.equal(compat.first_token_mask(idx, 128).cpu(), O.first_token_mask(idx.cpu(), 128))

@@ -29,3 +29,40 @@ def test_patched_model_matches_unpatched_on_gpu(dev, name):
     with torch.no_grad():
         lg = model2(ids).logits
     assert torch.isfinite(lg.float()).all()
+
+
+@pytest.mark.parametrize("method", ["pbs", "meanpooling", "dense"])
+def test_ttft_harness_writes_the_reference_result_record(dev, method, tmp_path, capsys):
+    """The offline harness follows eval/efficiency/eval_efficiency.py: one JSON line on stdout and a result
+    file <output_dir>/<method>_<len>.json with the fields of its results dict (:261-290)."""
+    import json
+    from pbs_attn_amd import ttft
+    argv = ["--method", method, "--layers", "2", "--len", "4096", "--iters", "2", "--warmup", "1",
+            "--output-dir", str(tmp_path)]
+    assert ttft.main(argv) == 0
+    line = capsys.readouterr().out.strip().splitlines()[-1]
+    printed = json.loads(line)
+    path = tmp_path / f"{method}_4096.json"
+    assert printed["result_file"] == str(path) and path.exists()
+    saved = json.loads(path.read_text())
+    for key in ("script_args", "method_args", "model_name", "tokenizer_name", "num_tokens", "avg_e2e_latency", "e2e_std"):
+        assert key in saved, key
+    assert saved["num_tokens"] == 4096 and saved["model_name"] == "llama31_8b"
+    assert saved["script_args"]["method"] == method and saved["script_args"]["len"] == 4096
+    assert saved["script_args"]["n_examples"] == 2 and saved["script_args"]["num_warmup_iter"] == 1
+    assert len(saved["e2e_latencies"]) == 2 and all(t > 0 for t in saved["e2e_latencies"])
+    assert abs(saved["avg_e2e_latency"] - sum(saved["e2e_latencies"]) / 2) < 1e-9
+    assert printed["ttft_s"] == saved["avg_e2e_latency"]
+    if method == "dense":
+        assert saved["method_args"] == {}
+    else:
+        assert saved["method_args"]["segment_size"] == (256 if method == "pbs" else 1024)
+        assert saved["method_args"]["threshold"] == 0.9 and saved["method_args"]["block_size"] == 128
+
+
+def test_ttft_harness_defaults_follow_the_protocol():
+    """30 warm-up generations and 10 examples unless overridden (eval_efficiency.py:36-37)."""
+    import inspect
+    from pbs_attn_amd import ttft
+    src = inspect.getsource(ttft.main)
+    assert 'default=30, dest="num_warmup_iter"' in src and 'default=10, dest="n_examples"' in src

@@ -130,9 +130,13 @@ def _oracle_selection(P_scores, thr, idx_pad, nb, bps, force_first):
 
 @pytest.mark.parametrize("nb,bps,thr,force_first", [
     (8, 2, 0.9, True), (32, 2, 0.8, True), (32, 8, 0.95, False), (40, 8, 1.0, True), (40, 8, 1, True),
-    (33, 1, 0.5, True), (100, 4, 0.0, True), (64, 2, "tensor", True), (300, 8, 0.9, True), (1030, 8, 0.9, True)])
+    (33, 1, 0.5, True), (100, 4, 0.0, True), (64, 2, "tensor", True), (300, 8, 0.9, True), (1030, 8, 0.9, True),
+    # config 4's row length (512 blocks) and config 2's (1024: every lane and register of the wave kernel live)
+    (512, 2, 0.9, True), (1024, 8, 0.9, True), (1024, 8, "tensor", False),
+    # the workgroup-per-row kernel (more than 1024 blocks): wave-parallel running sum
+    (1100, 8, 0.95, True), (2100, 8, "tensor", True)])
 def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
-    B, H, S = 2, 3, nb * 128 - 5
+    B, H, S = (2, 3, nb * 128 - 5) if nb <= 512 else (1, 2, nb * 128 - 5)
     g = torch.Generator().manual_seed(nb * 7 + bps)
     cand, _ = O.candidate_masks(nb, bps)
     # bf16-valued logits -> many exactly equal probabilities, as in the real path
@@ -159,6 +163,28 @@ def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
             for qb in qbs:
                 want = [kb for kb in range(nb) if ref_sel[b, h, qb, kb] and qseg[kb] < qseg[qb]]
                 assert cols[b, h, qb, :cnt[b, h, qb]].tolist() == want
+
+
+def test_select_blocks_threshold_kinds_follow_the_reference(dev):
+    # True is the int-1 rule there (isinstance(True, int)); a float64 tensor makes the compare a float64 one
+    nb, bps = 24, 4
+    g = torch.Generator().manual_seed(5)
+    cand, segm = O.candidate_masks(nb, bps)
+    Pm = torch.softmax((torch.randn((1, 2, nb, nb), generator=g) * 2).bfloat16().float().masked_fill(~cand, float("-inf")), -1)
+    idx_pad = torch.arange(nb * 128).expand(1, 2, -1).int()
+    args = (idx_pad.to(dev), nb * 128, 128, bps * 128, False)
+    sel_true, _, _, _ = ops.select_blocks(None, True, *args)
+    assert torch.equal(sel_true.cpu(), cand.expand(1, 2, -1, -1))
+    # thresholds chosen ON prefix sums: float32(prefix) >= float32(t) holds, float64 compare with the exact
+    # float64 value of the same number may not -- the oracle applies torch's promotion, the kernel must agree
+    srt = torch.sort(torch.nan_to_num(Pm, nan=0.0), -1, descending=True).values
+    pre = torch.cumsum(srt.double(), -1).float()[0, :, nb - 1, 2]          # one prefix per head
+    t64 = pre.double().view(1, 2) + 1e-9                                    # just above a reachable float32 prefix
+    got64, _, _, _ = ops.select_blocks(Pm.to(dev), t64.to(dev), *args)
+    assert torch.equal(got64.cpu(), O.select_blocks(Pm, t64))
+    got32, _, _, _ = ops.select_blocks(Pm.to(dev), t64.float().to(dev), *args)
+    assert torch.equal(got32.cpu(), O.select_blocks(Pm, t64.float()))
+    assert not torch.equal(got64.cpu(), got32.cpu())                        # the dtype of the tensor matters
 
 
 def test_select_blocks_nan_rows_and_zero_rows(dev):
@@ -216,6 +242,30 @@ def test_sparse_attention_strided_query(dev):
     buf = torch.empty((2, 768, 4, 128), dtype=q.dtype, device=dev).transpose(1, 2)
     ops.sparse_attn_fwd(q_strided, *args, out=buf)
     assert torch.equal(buf, out_c)
+
+
+def test_reference_naive_path_is_the_outlier_on_short_rows(dev):
+    """The reference's naive CPU path normalises the probabilities and THEN rounds them to bf16 (kernels/...:377-380);
+    its Triton kernel and this HIP kernel round the un-normalised probabilities and divide once at the end.  On
+    early rows, which attend to few keys, the first way loses more: on this input (seed 21, 768 tokens) the naive
+    path is farther from exact fp32 attention than the north-star tolerance, the HIP kernel is well inside it."""
+    q, k, v = small_case(2, 4, 2, 768, seed=21)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, 256, 0.9, return_intermediates=True)
+    idx_pad = mid["key_indices"].int().contiguous().to(dev)
+    kd, vd = k.to(dev), v.to(dev)
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx_pad, 4, want_orig_vt=True)
+    _, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), 0.9, idx_pad, 768, 128, 256, True)
+    assert torch.equal(fin.cpu(), mid["final_mask"])
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, orig_vt, cols, cnt, 256).cpu()
+    dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], mid["key_indices"], mid["final_mask"], 128)
+    hip_err = (out.float() - dense).abs()
+    naive_err = (ref.float() - dense).abs()
+    assert hip_err.max().item() <= 1e-2 and hip_err.mean().item() <= 1e-3          # half the tolerance
+    assert naive_err.max().item() > 2e-2                                            # the reference's own path is outside
+    assert naive_err.mean().item() <= 2e-3
+    # HIP vs naive therefore inherits the naive path's error: documented, not a HIP defect
+    assert (out.float() - ref.float()).abs().max().item() <= naive_err.max().item() + hip_err.max().item()
 
 
 # ---------------------------------------------------------------- whole pipeline on the GPU
@@ -279,17 +329,29 @@ def test_ones_value_rows_sum_to_one(dev):
     assert torch.allclose(out.float().cpu(), torch.ones(1, 2, 1536, 128), atol=8e-3)
 
 
-def test_end_to_end_matches_oracle_when_selection_agrees(dev):
-    # full HIP pipeline vs full oracle pipeline; they can only differ where a score
-    # near-tie flips the permutation, so compare where both chose the same key order
-    q, k, v = small_case(1, 4, 2, 2048, seed=12)
+def test_end_to_end_matches_oracle_where_the_selection_agrees(dev):
+    """Full HIP pipeline vs full oracle pipeline from raw Q, K, V.  The two can only differ where a near-tie of
+    the GPU-computed scores flips the permutation or the selection; the agreement is measured and every
+    query-block row with the same mask and the same key order up to its segment meets the output tolerance."""
+    B, H, S, seg = 1, 4, 2048, 256
+    q, k, v = small_case(B, H, 2, S, seed=12)
     ke, ve = expand_kv(q, k), expand_kv(q, v)
-    ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, 256, 0.9, return_intermediates=True)
-    out = P.permuted_block_sparse_attn_fwd(q.to(dev), k.to(dev), v.to(dev), 128, 256, 0.9, True).cpu()
-    diff = (out.float() - ref.float()).abs()
-    # thresholded selection drops ~10 % of the mass: different but equally valid selections
-    # still agree to that order; identical selections agree to bf16 tolerance
-    assert diff.mean().item() < 2e-2
+    ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, seg, 0.9, return_intermediates=True)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    perm = P.apply_permutation(qd, kd, vd, 128, seg)
+    sel = P.permuted_block_selection(qd, perm, 128, seg, 0.9)
+    out = perm.attention(qd, sel["csr_cols"], sel["csr_cnt"], seg).cpu()
+    same_idx = perm.key_indices.cpu()[:, :, :S].long() == mid["key_indices"]
+    same_mask = sel["final_mask"].cpu() == mid["final_mask"]
+    assert same_idx.float().mean().item() >= 0.99 and same_mask.float().mean().item() >= 0.99
+    nb, bps = S // 128, seg // 128
+    seg_same = same_idx.view(B, H, nb // bps, seg).all(-1)
+    prefix_same = torch.cumprod(seg_same.int(), dim=-1).bool().repeat_interleave(bps, dim=-1)
+    comparable = same_mask.all(-1) & prefix_same
+    diff = (out.float() - ref.float()).abs().view(B, H, nb, 128, 128)
+    assert comparable.float().mean().item() >= 0.5
+    assert diff.amax(dim=(-1, -2))[comparable].max().item() <= 2e-2
+    assert diff.mean(dim=(-1, -2))[comparable].mean().item() <= 2e-3
     assert torch.isfinite(out.float()).all()
 
 
