@@ -7,12 +7,16 @@ synthetic Llama-3.1-8B-shaped attention layer already resident in HBM.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2]
 
-prints ONE JSON line.  `value` is the effective TFLOP/s of the whole pass
-(4 * 128 * 128 * 128 FLOP per visited block pair / step time); `roofline` prices
-the dominant kernel (the block-sparse attention) against the bf16 dense MFMA peak
-with its duration taken from HIP events recorded around it inside the timed steps;
-`cpu_baseline` times the CPU restatement of the reference's torch path on a bounded
-sample on this host's cores.
+prints ONE JSON line.  The K timed steps are K calls of the operator as a caller
+makes them (`permuted_block_sparse_attn_fwd`, one library call each); `value` is the
+effective TFLOP/s of that pass (4 * 128 * 128 * 128 FLOP per visited block pair /
+step time).  A second, untimed-for-`value` pass runs the same work stage by stage with
+a HIP event after every stage: `stage_ms`, and `roofline`, which prices the dominant
+kernel (the block-sparse attention) against the bf16 dense MFMA peak.  `cpu_baseline`
+times the CPU restatement of the reference's torch path on a bounded sample on this
+host's cores.  The default run adds two more measurements as extra keys: `cfg1` (the
+32k layer: segment 256, threshold 0.9) and `ttft_llama31_8b_64k` (time to first token
+of the 32-layer architecture on a 64k prompt, patched against unpatched).
 """
 from __future__ import annotations
 
@@ -29,9 +33,22 @@ sys.path.insert(0, ROOT)
 PEAK_BF16_TFLOPS = 2500.0      # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 FLOP_PER_BLOCK_PAIR = 4.0 * 128 * 128 * 128
-# HBM bytes per launch of the attention kernel (fetched + written past L2), from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE scaled by a 1 GiB copy (profiles/pipeline_cfg2_hbm_traffic.txt); only known for that workload.
-MEASURED_ATTN_TRAFFIC_BYTES = {("cfg2", None, 1024, 0.9): 20.37e9 + 1.07e9}
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE summary of the default workload; the attention kernel's HBM bytes per
+# launch are read from its "traffic_bytes_per_launch" line when the run is that workload
+TRAFFIC_PROFILE = "profiles/pipeline_cfg2_hbm_traffic.txt"
+
+
+def measured_traffic(workload, kind, segment, threshold):
+    """(bytes per launch, source file) of sparse_attn_kernel from the committed counter summary, or (None, None)."""
+    import re
+    if (workload, kind, segment, threshold) != ("cfg2", None, 1024, 0.9):
+        return None, None
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            m = re.search(r"^traffic_bytes_per_launch\s+sparse_attn_kernel\s+([0-9.eE+]+)\s*$", f.read(), re.M)
+    except OSError:
+        return None, None
+    return (float(m.group(1)), TRAFFIC_PROFILE) if m else (None, None)
 
 
 def log(*a):
@@ -167,18 +184,32 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     def step():
         return P.permuted_block_sparse_attn_fwd(q, k, v, bs, seg, thr, True)
 
+    # the timed region: the operator as a caller makes it (no profiling hook: one library call per step)
+    assert P.stage_timer is None
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
-    timer = StageTimer(torch)
-    P.stage_timer = timer
     t0 = time.perf_counter()
     for _ in range(steps):
-        timer.begin()
         out = step()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / steps
-    P.stage_timer = None
+    # the same work stage by stage, a HIP event on the launch stream after every stage
+    timer = StageTimer(torch)
+    P.stage_timer = timer
+    try:
+        timer.begin()
+        step()
+        torch.cuda.synchronize()
+        timer.steps.clear()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            timer.begin()
+            out = step()
+        torch.cuda.synchronize()
+        staged_ms = (time.perf_counter() - t0) * 1e3 / steps
+    finally:
+        P.stage_timer = None
     stages = timer.summary()
 
     # visited block pairs of this input (one extra selection pass, outside the timed region)
@@ -191,7 +222,7 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     res = {
         "workload": name, "B": B, "Hq": Hq, "Hkv": Hkv, "S": S, "D": D, "block": bs, "segment": seg,
         "threshold": thr, "generator": cfg["kind"], "seed": seed,
-        "ms_per_step": wall_ms, "stage_ms": stages, "visited_block_pairs": n_vis,
+        "ms_per_step": wall_ms, "ms_per_step_staged": staged_ms, "stage_ms": stages, "visited_block_pairs": n_vis,
         "reference_block_pairs": n_ref,
         "density_vs_causal": n_vis / causal_pairs,
         "effective_tflops_pipeline": flops / (wall_ms * 1e-3) / 1e12,
@@ -241,18 +272,45 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     return res, (cfg, q, k, v)
 
 
-def density_without_permutation(torch, cfg, q, k, v):
-    """Block density of the same selection rule on UN-permuted keys (identity order through the same
-    kernels: strictly decreasing injected scores), the ablation that shows what the permutation buys."""
-    from pbs_attn_amd import pbs as P
-    B, Hq, S = cfg["B"], cfg["Hq"], cfg["S"]
-    bs, seg, thr = cfg["block"], cfg["segment"], cfg["threshold"]
-    sc = (S // seg) * seg
-    scores = -torch.arange(sc, device=q.device, dtype=torch.float32).view(1, 1, sc).expand(B, Hq, sc).contiguous()
-    perm = P.apply_permutation(q, k, v, bs, seg, scores=scores)
-    sel = P.permuted_block_selection(q, perm, bs, seg, thr, want_masks=False)
+def meanpooling_mode(torch, cfg, q, k, v, reps=2):
+    """The reference's MeanPooling baseline on the same tensors (`get_meanpooling_prefill`: PBS without the
+    permutation; same block size and threshold): block density of its mask and the time of one pass."""
+    from pbs_attn_amd.meanpooling import MeanPooling_prefill
+    B, Hq, S, bs, thr = cfg["B"], cfg["Hq"], cfg["S"], cfg["block"], cfg["threshold"]
     nb = (S + bs - 1) // bs
-    return block_pair_counts(sel["csr_cnt"], B, Hq, nb, seg // bs)[0] / (B * Hq * nb * (nb + 1) // 2)
+    _, mid = MeanPooling_prefill(q, k, v, bs, cfg["segment"], thr, return_masks=True)
+    pairs = int(mid["csr_cnt"].sum().item()) + B * Hq * nb          # selected earlier blocks + the diagonal block
+    del mid
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        MeanPooling_prefill(q, k, v, bs, cfg["segment"], thr)
+    e1.record()
+    torch.cuda.synchronize()
+    return pairs / (B * Hq * nb * (nb + 1) // 2), e0.elapsed_time(e1) / reps
+
+
+def ttft_pair(torch, length=65536, runs=3, warmup=1, model_name="llama31_8b", layers=None):
+    """Time to first token of the random-init architecture on a `length`-token prompt of uniform random ids:
+    the unpatched model (torch SDPA) and the same model patched with the PBS prefill (defaults: block 128,
+    segment 256, threshold 0.9).  `runs` timed generations each after `warmup` untimed ones."""
+    import contextlib
+    from pbs_attn_amd import ttft
+    from pbs_attn_amd.patch.huggingface import apply_patch_with_prefill, get_permuted_block_sparse_attn_fwd
+    t0 = time.perf_counter()
+    model = ttft.build_model(model_name, layers)
+    out = {"model": model_name, "layers": model.config.num_hidden_layers, "num_tokens": length, "runs": runs,
+           "warmup": warmup, "weights": "random init", "prompts": "uniform random token ids", "unit": "s"}
+    dense = ttft.measure(model, length, warmup, runs)
+    with contextlib.redirect_stdout(sys.stderr):
+        apply_patch_with_prefill(model, get_permuted_block_sparse_attn_fwd())
+    pbs = ttft.measure(model, length, warmup, runs)
+    out.update(pbs_s=sum(pbs) / runs, dense_s=sum(dense) / runs, pbs_runs=pbs, dense_runs=dense,
+               speedup_vs_dense=sum(dense) / sum(pbs), wall_s=time.perf_counter() - t0)
+    del model
+    torch.cuda.empty_cache()
+    return out
 
 
 def run_report(torch, path, steps, warmup):
@@ -261,20 +319,21 @@ def run_report(torch, path, steps, warmup):
     runs += [("cfg1", {"segment": sg, "threshold": th}) for sg in (256, 1024) for th in (0.8, 0.9, 0.95)
              if not (sg == 256 and th == 0.9)]
     runs += [("cfg2", {}), ("cfg3", {}), ("cfg3", {"segment": 1024}),
-             ("cfg1", {"kind": "strong_heavy", "segment": 1024}), ("cfg2", {"kind": "strong_heavy"})]
-    lines = ["| workload | generator | S | B x Hq/Hkv | segment | thr | density | density w/o permutation | pass ms | "
+             ("cfg1", {"kind": "strong_heavy", "segment": 1024}), ("cfg2", {"kind": "strong_heavy"}),
+             ("cfg2", {"kind": "strong_uniform"})]
+    lines = ["| workload | generator | S | B x Hq/Hkv | segment | thr | density | MeanPooling density | MeanPooling ms | pass ms | "
              "attn ms | attn TFLOP/s | % MFMA peak | dense SDPA ms | speed-up vs dense | score/sort/gather/estimate/select ms |",
-             "|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|"]
+             "|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|"]
     out = []
     for name, ov in runs:
         res, (cfg, q, k, v) = run_workload(torch, name, steps, warmup, overrides=ov, with_dense=True)
-        res["density_unpermuted"] = density_without_permutation(torch, cfg, q, k, v)
+        res["density_unpermuted"], res["meanpooling_ms"] = meanpooling_mode(torch, cfg, q, k, v)
         del q, k, v
         torch.cuda.empty_cache()
         st = res["stage_ms"]
         lines.append(
             f"| {name} | {res['generator']} | {res['S']} | {res['B']} x {res['Hq']}/{res['Hkv']} | {res['segment']} | "
-            f"{res['threshold']} | {res['density_vs_causal']:.3f} | {res['density_unpermuted']:.3f} | {res['ms_per_step']:.2f} | "
+            f"{res['threshold']} | {res['density_vs_causal']:.3f} | {res['density_unpermuted']:.3f} | {res['meanpooling_ms']:.2f} | {res['ms_per_step']:.2f} | "
             f"{st['sparse_attn']:.2f} | {res['effective_tflops_attn_kernel']:.0f} | "
             f"{100 * res['effective_tflops_attn_kernel'] / PEAK_BF16_TFLOPS:.1f} | "
             f"{res['dense_sdpa_ms']:.2f} | {res['dense_sdpa_ms'] / res['ms_per_step']:.2f} | "
@@ -299,6 +358,8 @@ def main():
     ap.add_argument("--no-dense", action="store_true")
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only ceiling measurement")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
+    ap.add_argument("--no-extras", action="store_true",
+                    help="skip the two extra measurements of the default run (the 32k layer and the 64k time to first token)")
     ap.add_argument("--report", default=None, metavar="FILE.md",
                     help="run every single-layer configuration and the sweeps, write a markdown table, and exit")
     ap.add_argument("--traffic-calibration", action="store_true",
@@ -341,6 +402,7 @@ def main():
 
     attn_s = res["stage_ms"]["sparse_attn"] * 1e-3
     achieved = res["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / attn_s / 1e12
+    traffic, traffic_source = measured_traffic(args.workload, args.kind, res["segment"], res["threshold"])
     line = {
         "metric": "pbs_prefill_attn_effective_tflops",
         "value": res["effective_tflops_pipeline"],
@@ -357,10 +419,10 @@ def main():
                    "reference_block_pairs": res["reference_block_pairs"]},
         "roofline": {"bound": "mfma", "kernel": "sparse_attn_kernel", "achieved": achieved, "peak": PEAK_BF16_TFLOPS,
                      "unit": "TFLOP/s", "frac": achieved / PEAK_BF16_TFLOPS,
-                     "traffic": MEASURED_ATTN_TRAFFIC_BYTES.get((args.workload, args.kind, res["segment"], res["threshold"])),
-                     "traffic_unit": "bytes/launch",
+                     "traffic": traffic, "traffic_unit": "bytes/launch", "traffic_source": traffic_source,
                      "kernel_ms": res["stage_ms"]["sparse_attn"]},
         "stage_ms": res["stage_ms"],
+        "ms_per_step_staged": res["ms_per_step_staged"],
         "hbm_gbs": res["hbm_gbs"],
         "dense_sdpa_ms": res.get("dense_sdpa_ms"),
         "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
@@ -374,6 +436,24 @@ def main():
         line["roofline"]["kernel_ms_zero_operands"] = res["attn_ms_zero_operands"]
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(*inputs, seconds_budget=args.cpu_seconds)
+    del inputs
+    torch.cuda.empty_cache()
+    if not (args.no_extras or overrides or args.workload != "cfg2"):
+        # the other two figures the headline metric names, measured the same way in the same run
+        r1, inputs1 = run_workload(torch, "cfg1", max(args.steps, 10), max(args.warmup, 3))
+        del inputs1
+        torch.cuda.empty_cache()
+        log("[bench] cfg1 " + json.dumps(r1))
+        a1 = r1["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / (r1["stage_ms"]["sparse_attn"] * 1e-3) / 1e12
+        line["cfg1"] = {
+            "workload": f"cfg1: same layer shape, S={r1['S']}, block {r1['block']}, segment {r1['segment']}, threshold "
+                        f"{r1['threshold']}, generator {r1['generator']} seed {r1['seed']}",
+            "ms_per_step": r1["ms_per_step"], "value": r1["effective_tflops_pipeline"], "unit": "TFLOP/s",
+            "density_vs_causal": r1["density_vs_causal"], "stage_ms": r1["stage_ms"],
+            "attn_kernel_tflops": a1, "attn_kernel_frac_of_peak": a1 / PEAK_BF16_TFLOPS,
+            "dense_sdpa_ms": r1.get("dense_sdpa_ms"), "speedup_vs_dense_sdpa": r1.get("speedup_vs_dense_sdpa")}
+        line["ttft_llama31_8b_64k"] = ttft_pair(torch)
+        log("[bench] ttft " + json.dumps(line["ttft_llama31_8b_64k"]))
     print(json.dumps(line), flush=True)
 
 

@@ -17,6 +17,10 @@ workloads
 ``strong_heavy``    ``uniform_heavy`` with a 10x stronger signal (K += 30u,
                     Q += 15u) clustered in spans: the supplementary input on
                     which permutation visibly raises block sparsity.
+``strong_uniform``  the 10x signal on 2 % of the key positions drawn uniformly (no spans):
+                    every 128-key block holds a few heavy keys, so without the
+                    permutation no block stands out; sorting inside a segment moves
+                    them into the segment's first block.
 """
 from __future__ import annotations
 
@@ -51,10 +55,10 @@ def make_qkv(B, Hq, Hkv, S, D, kind="uniform_heavy", seed=0, device="cpu", dtype
     u = _unit((B, Hkv, D), gen, device)
 
     heavy = torch.zeros(S, dtype=torch.bool)
-    if kind in ("uniform_heavy", "local_window"):
+    if kind in ("uniform_heavy", "local_window", "strong_uniform"):
         n = max(1, int(round(0.02 * S)))
         heavy[torch.randperm(S, generator=pos_gen)[:n]] = True
-        kq_gain = (3.0, 1.5)
+        kq_gain = (30.0, 15.0) if kind == "strong_uniform" else (3.0, 1.5)
     elif kind in ("span_heavy", "strong_heavy"):
         n_spans = min(64, max(1, S // 128))
         span = max(1, int(round(0.01 * S / n_spans)))

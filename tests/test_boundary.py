@@ -276,7 +276,7 @@ def test_synthetic_generators_are_seeded_and_shaped():
     b = make_qkv(1, 4, 2, 256, 128, "uniform_heavy", seed=5)
     assert all(torch.equal(x, y) for x, y in zip(a, b))
     assert a[0].shape == (1, 4, 256, 128) and a[1].shape == (1, 2, 256, 128) and a[0].dtype == torch.bfloat16
-    for kind in ("span_heavy", "local_window", "strong_heavy"):
+    for kind in ("span_heavy", "local_window", "strong_heavy", "strong_uniform"):
         q, k, v = make_qkv(2, 4, 1, 640, 128, kind, seed=1)
         assert q.shape == (2, 4, 640, 128) and torch.isfinite(q.float()).all()
     assert set(WORKLOADS) >= {"cfg0", "cfg1", "cfg2", "cfg3"}
