@@ -111,13 +111,17 @@ int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per
  * query sees are exactly those of the reference's final mask and element mask
  * (a segment's permuted blocks hold the same keys as its original blocks).
  * out: (B, Hq, S, 128) bf16 with its own strides, original query order.
+ * workspace: pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size) bytes of device memory, 256-byte
+ * aligned (work counters and the merged visit list of every pair of query blocks, rewritten by each call).
+ * Two launches: the list merge, then one persistent workgroup per CU.
  * Replaces pbs_attn/src/kernels/permuted_block_sparse_attention.py:134-311
  * (launch at pbs_attn/src/pbs.py:220-246). */
+size_t pbs_sparse_attn_workspace_bytes(int B, int Hq, int S, int segment_size);
 int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
                         const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
                         int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
                         int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                        float softmax_scale, void* stream);
+                        float softmax_scale, void* workspace, void* stream);
 
 /* out[b,h,q_idx[b,h,i],:] = o_perm[b,h,i,:] (o_perm contiguous).  q_idx null with
  * o_perm == out is the identity fast path (no launch): the reference does not

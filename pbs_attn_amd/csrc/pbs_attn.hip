@@ -8,12 +8,20 @@
 //     on key order, so this is the reference's "every block of the own segment, element mask original key
 //     position > query position" with half the tiles and one masked tile instead of all.
 // Work decomposition
-//   One workgroup (8 waves, two per SIMD) owns TWO adjacent 128-query blocks of one head.  Waves
-//   0-3 serve the first block, waves 4-7 the second, 32 queries per wave.  The two visit lists
-//   (ascending key-block indices) are merged once into LDS, the own-segment blocks appended; every merged
-//   tile is copied ONCE into LDS for both query blocks, which halves the L2 -> LDS traffic and doubles
-//   the time a tile stays in flight.  K and V tiles are double-buffered (2 x 64 KB) and fetched one tile
-//   ahead with asynchronous global -> LDS copies (no registers), one workgroup barrier per tile.
+//   A work item is TWO adjacent 128-query blocks of one head, served by one workgroup (8 waves, two per
+//   SIMD): waves 0-3 take the first block, waves 4-7 the second, 32 queries per wave.  A small kernel
+//   first merges the two visit lists of every item (ascending key-block indices, own-segment blocks
+//   appended) into one list in HBM; every merged tile is copied ONCE into LDS for both query blocks, which
+//   halves the L2 -> LDS traffic and doubles the time a tile stays in flight.  K and V tiles are
+//   double-buffered (2 x 64 KB) and fetched one tile ahead with asynchronous global -> LDS copies (no
+//   registers), one workgroup barrier per tile.
+//   The attention kernel is PERSISTENT: one workgroup per CU takes item after item from a counter (one per
+//   XCD, over that XCD's share of the items; when it runs dry, the other XCDs' counters).  The tile pipeline
+//   runs across items: the next item is claimed three tiles before the end of the current one, its list and
+//   its queries (into L2) are requested one tile later, its first K / V tiles at the last tile, so that an
+//   item's fixed costs (list, first tile, write-out of the previous item) overlap attention work.  With short
+//   visit lists (a few tiles per item) that is the difference between waiting for HBM three times per item
+//   and once.
 // Data layout
 //   K tile: 128 keys x 128 d row-major; V tile: stored TRANSPOSED in HBM by the gather kernel,
 //   128 d x 128 keys.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
@@ -27,7 +35,7 @@
 //   the unrounded values; the output is normalised once at the end.
 // Tile kinds
 //   * fast tiles: a software pipeline over the four 32-key sub-tiles -- S of sub-tile k+1, exponentials
-//     of sub-tile k and P.V of sub-tile k-1 are issued interleaved, LDS fragments are read three slots
+//     of sub-tile k and P.V of sub-tile k-1 are issued interleaved, LDS fragments are read two slots
 //     ahead.  Exponentials are taken against a LAZY reference maximum: it is not updated per tile; a row
 //     sum of one tile above 2^14 triggers a uniform rescale (exact, all terms share the reference); an
 //     overflow marks the row and the whole workgroup redoes it without speculation.  The first tile of a
@@ -45,12 +53,14 @@ constexpr int D = 128;
 constexpr int BS = 128;
 constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
 constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
-constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // merged visit list, uint16 entries (<= 4096 + 1)
-constexpr uint32_t LDS_MISC = LDS_LIST + 10240;   // ints: [0] merged count, [1] redo flag, [16..24) wave totals
-constexpr uint32_t LDS_TOTAL = LDS_MISC + 1024;   // 142 336 bytes of the CU's 160 KB
+constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // two merged visit lists (current item, next item), uint16 entries
+constexpr uint32_t LIST_BYTES = 9728;             // count + at most 4096 + 511 + 1 entries, rounded up
+constexpr uint32_t LDS_MISC = LDS_LIST + 2 * LIST_BYTES;   // ints: [1] redo flag, [2] first work item, [4] next work item
+constexpr uint32_t LDS_DUMP = LDS_MISC + 1024;    // 1 KB per wave: landing area of copies issued only to bring lines into L2
+constexpr uint32_t LDS_TOTAL = LDS_DUMP + 8192;   // 159 744 bytes of the CU's 160 KB
 constexpr uint32_t ENT_KB = 0x1fffu;              // visit-list entry: key block ...
 constexpr uint32_t ENT_ORIG = 0x2000u;            // ... | tile of the un-permuted K / V (own segment) | use bits 14, 15
-constexpr int PREFETCH_SLOTS = 3;                 // LDS fragment reads run this many slots ahead
+constexpr int PREFETCH_SLOTS = 2;                 // LDS fragment reads run this many slots ahead
 
 struct AttnArgs {
   const uint16_t* q;
@@ -58,8 +68,9 @@ struct AttnArgs {
   const uint16_t* pvt;   // (B*Hq, nb, 128, 128) permuted V blocks, transposed
   const uint16_t* k;     // original K at the KV heads, caller's strides
   const uint16_t* ovt;   // (B*Hkv, nb, 128, 128) original-order V blocks, transposed
-  const int32_t* cols;   // (B*Hq, nb, nb)
-  const int32_t* cnt;    // (B*Hq, nb)
+  const uint16_t* plist; // (B*Hq * npair, cap) merged visit lists
+  int* queue;            // 8 work counters, one per XCD
+  int cap;               // entries per list row (multiple of 8)
   uint16_t* o;
   int BH, Hq, Hkv, S, nb, bps;
   uint32_t k_ss;   // key row stride in elements (< 2^22)
@@ -69,6 +80,15 @@ struct AttnArgs {
 };
 
 typedef __attribute__((address_space(3))) uint8_t lds_u8;
+typedef const __attribute__((address_space(4))) struct AttnArgs* ArgsPtr;
+
+// lane id formed where it is asked for: as a plain intrinsic it is computed once at the top of the kernel and
+// everything derived from it holds registers from there on
+__device__ __forceinline__ int lane_id_here() {
+  int l;
+  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
+  return l;
+}
 
 // row of the 32-row MFMA tile -> key of the 32-key sub-tile, chosen so that the accumulator
 // registers 8u..8u+7 of lane-half g hold keys 16u + 8g + 0..7
@@ -152,14 +172,17 @@ __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
 // (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
 // query: key-in-tile > query-in-block, an arithmetic test.
 template <bool MASKED, int PF>
-__device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t (&koff)[8],
-                                          const uint32_t (&voff)[8], uint32_t bufx, float c_log2, float& m_ref,
-                                          float& l_part, bool& poisoned, int wq, int j, int gh) {
+__device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t koff0,
+                                          const uint32_t voff0, const uint32_t (&bx)[8], float c_log2, float& m_ref,
+                                          float& l_part, bool& poisoned, int wq) {
   // query-in-block minus the lane half's key offset; made opaque per call: the 128 mask compares of a
   // diagonal tile depend only on the lane, and hoisted out of the tile loop they would each pin a 64-bit
   // scalar mask
-  int qrel8 = 32 * wq + j - 8 * gh;
-  if (MASKED) asm volatile("" : "+v"(qrel8));
+  int qrel8 = 0;
+  if (MASKED) {
+    const int ln = lane_id_here();          // nothing below may be formed outside the tile
+    qrel8 = 32 * wq + (ln & 31) - 8 * (ln >> 5);
+  }
   const float negm = -m_ref;
   float rsum[4] = {0.f, 0.f, 0.f, 0.f};
   f32x16 sbuf[2];
@@ -167,14 +190,14 @@ __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8],
   constexpr int R = PF + 1;
   bf16x8 frk[R], frv[R];
 #pragma unroll
-  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf((koff[n & 7] ^ bufx) + (n >> 3) * 8192);
+  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf((koff0 ^ bx[n & 7]) + (n >> 3) * 8192);
 #pragma clang loop unroll(full)
   for (int n = 0; n < 48; ++n) {
     const int step = n >> 3, t = n & 7;
     {   // fragment reads for slot n + PF
       const int m = n + PF, mstep = m >> 3, mt = m & 7;
-      if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff[mt] ^ bufx) + mstep * 8192);
-      if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff[2 * (mstep - 2) + (mt >> 2)] ^ bufx) + (mt & 3) * 8192);
+      if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff0 ^ bx[mt]) + mstep * 8192);
+      if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff0 ^ bx[2 * (mstep - 2) + (mt >> 2)]) + (mt & 3) * 8192);
     }
     if (step <= 3) {
       const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
@@ -218,298 +241,496 @@ __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8],
   }
 }
 
+// ---- merged visit list of a pair of query blocks, built once per pass by its own kernel:
+// row (bh * npair + pair) of `plist`: [0] = number of tiles, [1 ..] = entries kb | ENT_ORIG? | use_first << 14 |
+// use_second << 15: the union of the two visit lists (ascending), then the own segments in ORIGINAL key order
+// (blocks first-of-segment .. query block, shared where the two blocks share a segment).  Block 0 also clears
+// the work counters of the attention kernel that follows on the stream.
+__global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __restrict__ cols, const int32_t* __restrict__ cnt,
+                                                               uint16_t* __restrict__ plist, int* __restrict__ queue, int nb,
+                                                               int bps, int cap) {
+  __shared__ uint8_t flags0[4096], flags1[4096];
+  __shared__ int wsum[8];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int npair = (nb + 1) >> 1;
+  const int bh = blockIdx.x / npair, pair = blockIdx.x % npair;
+  if (blockIdx.x == 0 && tid < 8) queue[tid] = 0;
+  const bool second = 2 * pair + 1 < nb;
+  const int32_t* l0 = cols + ((int64_t)bh * nb + 2 * pair) * nb;
+  const int32_t* l1 = l0 + (second ? nb : 0);
+  const int n0 = cnt[(int64_t)bh * nb + 2 * pair];
+  const int n1 = second ? cnt[(int64_t)bh * nb + 2 * pair + 1] : 0;
+  constexpr int MAX_PER = 4096 / 512;
+  int c0[MAX_PER], c1[MAX_PER];
+#pragma unroll
+  for (int u = 0; u < MAX_PER; ++u) {
+    const int i = tid + 512 * u;
+    c0[u] = i < n0 ? l0[i] : 0;
+    c1[u] = i < n1 ? l1[i] : 0;
+  }
+  for (int i = tid; i < nb; i += 512) {
+    flags0[i] = 0;
+    flags1[i] = 0;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int u = 0; u < MAX_PER; ++u) {
+    const int i = tid + 512 * u;
+    if (i < n0) flags0[c0[u]] = 1;
+    if (i < n1) flags1[c1[u]] = 2;
+  }
+  __syncthreads();
+  // compaction: thread t owns `per` consecutive key blocks; wave-level prefix, then wave totals
+  const int per = (nb + 511) / 512;
+  const int k0 = tid * per, k1 = min(k0 + per, nb);
+  int c = 0;
+  for (int kb = k0; kb < k1; ++kb) c += (flags0[kb] | flags1[kb]) ? 1 : 0;
+  int incl = c;
+#pragma unroll
+  for (int off = 1; off < 64; off <<= 1) {
+    const int up = __shfl_up(incl, off, 64);
+    if (lane >= off) incl += up;
+  }
+  if (lane == 63) wsum[wave] = incl;
+  __syncthreads();
+  int w = incl - c, total = 0;
+#pragma unroll
+  for (int x = 0; x < 8; ++x) {
+    const int ws = wsum[x];
+    if (x < wave) w += ws;
+    total += ws;
+  }
+  uint16_t* out = plist + (int64_t)blockIdx.x * cap;
+  for (int kb = k0; kb < k1; ++kb) {
+    const int f = flags0[kb] | flags1[kb];
+    if (f) out[1 + w++] = (uint16_t)(kb | (f << 14));
+  }
+  const int qb0 = 2 * pair, qb1 = second ? qb0 + 1 : qb0;
+  const int sf0 = (qb0 / bps) * bps, sf1 = (qb1 / bps) * bps;
+  const int n_own = qb1 - sf0 + 1;
+  if (tid < n_own) {
+    const int kb = sf0 + tid;
+    const int f = (kb <= qb0 ? 1 : 0) | ((second && kb >= sf1) ? 2 : 0);
+    out[1 + total + tid] = (uint16_t)(kb | ENT_ORIG | (f << 14));
+  }
+  if (tid == 0) out[0] = (uint16_t)(total + n_own);
+}
+
+// asynchronous copy of one list row (`chunks` 16-byte pieces) into LDS at byte offset `lds_byte`
+__device__ __forceinline__ void stage_list_async(const uint16_t* src, int chunks, uint32_t lds_byte, int wave, int tid) {
+  const uint64_t src0 = (uint64_t)(uintptr_t)src;
+  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
+  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
+  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
+  for (int p = 0; p * 512 < chunks; ++p) {
+    const int chunk = p * 512 + tid;
+    const uint32_t voff = (uint32_t)chunk * 16u;
+    if (chunk < chunks) {
+      register uint32_t m0v asm("m0") = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + p * 8192 + wave * 1024));
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu) : "memory");
+    }
+  }
+}
+
 __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // starts at LDS offset 0
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int j = lane & 31, gh = lane >> 5;
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int grp = wave >> 2, wq = wave & 3;
 
-  // workgroup -> (head, pair of query blocks).  The work items, ordered head by head with the long rows of
-  // a head first, are cut into eight contiguous ranges of about equal work, one per XCD (blockIdx % 8):
-  // an XCD works through one head at a time, so its resident workgroups walk the same permuted K/V
-  // stream at about the same pace and share its tiles in that XCD's L2; with fewer heads than XCDs, or
-  // a head count that is no multiple of 8, a head is split between XCDs instead of leaving some idle
-  const int npair = (a.nb + 1) >> 1;
-  const int w_id = blockIdx.x;
-  const int xcd = w_id & 7, slot_id = w_id >> 3;
-  const int item = a.xcd_start[xcd] + slot_id;
-  if (item >= a.xcd_start[xcd + 1]) return;
-  const int bh = item / npair;
-  const int pair = npair - 1 - item % npair;
-  if (bh >= a.BH) return;
-  const int b = bh / a.Hq, h = bh % a.Hq;
-  const int qb = 2 * pair + grp;
-  const bool qb_valid = qb < a.nb;
-  const int qpos = qb * BS + 32 * wq + j;
-
-  uint16_t* mlist = reinterpret_cast<uint16_t*>(smem + LDS_LIST);
-  int* misc = reinterpret_cast<int*>(smem + LDS_MISC);
-
-  // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7.  Issued first so that the loads
-  // are in flight while the visit list is built.  Rows past the end of the sequence compute on the last
-  // row's values and are never stored.
-  bf16x8 qf[8];
-  {
-    const uint16_t* qrow = a.q + b * a.q_sb + h * a.q_sh + (int64_t)min(qpos, a.S - 1) * a.q_ss;
-#pragma unroll
-    for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(qrow + 16 * t + 8 * gh);
+  // Work items = (head, pair of query blocks), ordered head by head with the long rows of a head first and cut
+  // into eight contiguous ranges of about equal work, one per XCD (blockIdx % 8): an XCD works through one
+  // head at a time, so its resident workgroups walk the same permuted K/V stream at about the same pace and
+  // share its tiles in that XCD's L2.  The launch holds one workgroup per CU; each takes the next item of its
+  // XCD's range from a counter until the range is used up, so that the copies of an item's first tiles, the
+  // fetch of its list and of its queries overlap the previous item's last tile and epilogue.
+  // The arguments are read through the kernel-argument pointer where they are needed, and that pointer is made
+  // opaque once per item: scalar loads from it stay next to their use instead of pinning some fifty scalar
+  // registers for the whole kernel.
+#define PBS_ARGS() ({ ArgsPtr p_ = (ArgsPtr)__builtin_amdgcn_kernarg_segment_ptr(); asm volatile("" : "+s"(p_)); p_; })
+  ArgsPtr a0 = PBS_ARGS();
+  const int npair = (a0->nb + 1) >> 1;
+  const int xcd = blockIdx.x & 7;
+  int q_begin = a0->xcd_start[xcd], q_end = a0->xcd_start[xcd + 1];   // the range being served: this XCD's, later others'
+  int vic = xcd, vic_tried = 0;
+  int* misc = reinterpret_cast<int*>(smem + LDS_MISC);   // [1] redo flag, [2] first item, [4] next item
+  if (threadIdx.x == 0) {
+    misc[2] = q_begin + atomicAdd(a0->queue + xcd, 1);
+    misc[1] = 0;
   }
-
-  // ---- merged visit list of the two query blocks: entry = kb | use_first << 14 | use_second << 15.
-  // Counts and both column lists are fetched together (entries past a row's count are read and ignored).
-  {
-    uint8_t* flags0 = smem;          // nb bytes each; the tile area is free before the main loop
-    uint8_t* flags1 = smem + 4096;
-    const bool second = 2 * pair + 1 < a.nb;
-    const int32_t* l0 = a.cols + ((int64_t)bh * a.nb + 2 * pair) * a.nb;
-    const int32_t* l1 = l0 + (second ? a.nb : 0);
-    const int n0 = a.cnt[(int64_t)bh * a.nb + 2 * pair];
-    const int n1 = second ? a.cnt[(int64_t)bh * a.nb + 2 * pair + 1] : 0;
-    constexpr int MAX_PER = 4096 / 512;
-    int c0[MAX_PER], c1[MAX_PER];
-#pragma unroll
-    for (int u = 0; u < MAX_PER; ++u) {
-      const int i = tid + 512 * u;
-      c0[u] = i < a.nb ? l0[i] : 0;
-      c1[u] = i < a.nb ? l1[i] : 0;
-    }
-    for (int i = tid; i < a.nb; i += 512) {
-      flags0[i] = 0;
-      flags1[i] = 0;
-    }
-    if (tid == 0) misc[1] = 0;
-    __syncthreads();
-#pragma unroll
-    for (int u = 0; u < MAX_PER; ++u) {
-      const int i = tid + 512 * u;
-      if (i < n0) flags0[c0[u]] = 1;
-      if (i < n1) flags1[c1[u]] = 2;
-    }
-    __syncthreads();
-    // compaction: thread t owns `per` consecutive key blocks; wave-level prefix, then wave totals
-    const int per = (a.nb + 511) / 512;
-    const int k0 = tid * per, k1 = min(k0 + per, a.nb);
-    int c = 0;
-    for (int kb = k0; kb < k1; ++kb) c += (flags0[kb] | flags1[kb]) ? 1 : 0;
-    int incl = c;
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const int up = __shfl_up(incl, off, 64);
-      if (lane >= off) incl += up;
-    }
-    int* wsum = misc + 16;
-    if (lane == 63) wsum[wave] = incl;
-    __syncthreads();
-    int w = incl - c, total = 0;
-#pragma unroll
-    for (int x = 0; x < 8; ++x) {
-      const int ws = wsum[x];
-      if (x < wave) w += ws;
-      total += ws;
-    }
-    for (int kb = k0; kb < k1; ++kb) {
-      const int f = flags0[kb] | flags1[kb];
-      if (f) mlist[w++] = (uint16_t)(kb | (f << 14));
-    }
-    // then the own segments in ORIGINAL key order: blocks first-of-segment .. query block (causal), the
-    // same for both query blocks where they share a segment
-    const int qb0 = 2 * pair, qb1 = second ? qb0 + 1 : qb0;
-    const int sf0 = (qb0 / a.bps) * a.bps, sf1 = (qb1 / a.bps) * a.bps;
-    const int n_own = qb1 - sf0 + 1;
-    if (tid < n_own) {
-      const int kb = sf0 + tid;
-      const int f = (kb <= qb0 ? 1 : 0) | ((second && kb >= sf1) ? 2 : 0);
-      mlist[total + tid] = (uint16_t)(kb | ENT_ORIG | (f << 14));
-    }
-    if (tid == 0) misc[0] = total + n_own;
-    __syncthreads();
-  }
-  const int n_tiles = misc[0];
-
-  const uint16_t* pk = a.pk + (int64_t)bh * a.nb * BS * D;
-  const uint16_t* pvt = a.pvt + (int64_t)bh * a.nb * BS * D;
-  const int kvh = h / (a.Hq / a.Hkv);
-  const uint16_t* korig = a.k + b * a.k_sb + kvh * a.k_sh;
-  const uint16_t* ovt = a.ovt + (int64_t)(b * a.Hkv + kvh) * a.nb * BS * D;
-
-  // per-lane LDS byte offsets of the fragments inside buffer 0; XOR 0x8000 switches buffer.
-  //   K fragment (sub-tile ks, d-step t)      : koff[t] + ks * 8192
-  //   V fragment (keys 16 c .. 16 c + 15, dt) : voff[c] + dt * 8192
-  const int krow = mfma_row_to_key(j);
-  uint32_t koff[8], voff[8];
-#pragma unroll
-  for (int t = 0; t < 8; ++t) koff[t] = (uint32_t)(krow * 256 + (((2 * t + gh) ^ (krow & 15)) * 16));
-#pragma unroll
-  for (int c = 0; c < 8; ++c) voff[c] = LDS_V0 + (uint32_t)(j * 256 + (((2 * c + gh) ^ (j & 15)) * 16));
-  const uint32_t lane_off = async_lane_offset(wave, lane);
-  const float c_log2 = a.scale_log2;
-  // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf` (0 or 0x8000)
-  auto stage_entry = [&](uint32_t e, uint32_t buf) {
-    const int kb_e = (int)(e & ENT_KB);
-    if (e & ENT_ORIG) {
-      stage_krows_async(korig + (int64_t)kb_e * BS * a.k_ss, a.k_ss, a.S - kb_e * BS, buf, wave, lane);
-      stage_tile_async(ovt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
-    } else {
-      stage_tile_async(pk + (int64_t)kb_e * BS * D, buf, wave, lane_off);
-      stage_tile_async(pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
-    }
-  };
+  __syncthreads();
+  int cur = __builtin_amdgcn_readfirstlane(misc[2]);
+  if (cur >= q_end) return;
+  int nxt = q_end;   // the next item is claimed late in the current one: an item claimed early waits for this
+                     // workgroup while others may be idle
+  bool has_nxt = false;
   const uint32_t use_bit = 1u << (14 + grp);
 
-  for (int attempt = 0; attempt < 2; ++attempt) {
-    const bool careful_only = attempt == 1;
-    f32x16 o[4];
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt) o[dt] = (f32x16){0};
-    float m_ref = -INFINITY;   // reference maximum, identical in lanes j and j + 32
-    float l_part = 0.f;        // row sum of this lane's half of the keys
-    bool first = true, poisoned = false;
-    bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
+  // base pointers of one head's tiles: permuted K, permuted V^T, original K rows, original-order V^T
+  struct HeadBase {
+    const uint16_t *pk, *pvt, *korig, *ovt;
+    uint32_t k_ss;
+    int S;
+  };
+  auto head_base = [&](ArgsPtr ap, int bh_e) {
+    HeadBase hb;
+    const int Hq_e = ap->Hq, Hkv_e = ap->Hkv, nb_e = ap->nb;
+    const int b_e = bh_e / Hq_e, kvh = (bh_e % Hq_e) / (Hq_e / Hkv_e);
+    hb.pk = ap->pk + (int64_t)bh_e * nb_e * BS * D;
+    hb.pvt = ap->pvt + (int64_t)bh_e * nb_e * BS * D;
+    hb.korig = ap->k + b_e * ap->k_sb + kvh * ap->k_sh;
+    hb.ovt = ap->ovt + (int64_t)(b_e * Hkv_e + kvh) * nb_e * BS * D;
+    hb.k_ss = ap->k_ss;
+    hb.S = ap->S;
+    return hb;
+  };
+  // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf`
+  auto stage_entry = [&](const HeadBase& hb, uint32_t e, uint32_t buf, int lane, uint32_t lane_off) {
+    const int kb_e = (int)(e & ENT_KB);
+    if (e & ENT_ORIG) {
+      stage_krows_async(hb.korig + (int64_t)kb_e * BS * hb.k_ss, hb.k_ss, hb.S - kb_e * BS, buf, wave, lane);
+      stage_tile_async(hb.ovt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+    } else {
+      stage_tile_async(hb.pk + (int64_t)kb_e * BS * D, buf, wave, lane_off);
+      stage_tile_async(hb.pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+    }
+  };
+  auto list_row = [&](ArgsPtr ap, int item) {
+    const int bh_i = item / npair, pair_i = npair - 1 - item % npair;
+    return ap->plist + ((int64_t)bh_i * npair + pair_i) * ap->cap;
+  };
 
-    __syncthreads();   // list build / previous attempt are done with the tile buffers
-    stage_entry((uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[0]), 0u);   // the list is never empty
-    for (int it = 0; it < n_tiles; ++it) {
-      const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it]);
-      const int kb = (int)(ent & ENT_KB);
-      const bool has_next = it + 1 < n_tiles;
-      const uint32_t bufx = (it & 1) ? 0x8000u : 0u;
-      __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` has landed
-      __syncthreads();                      // every share has; every wave is done with tile it - 1
-      if (has_next) stage_entry((uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[it + 1]), bufx ^ 0x8000u);
-      if (!(ent & use_bit) || !qb_valid) continue;
-      const bool masked = (ent & ENT_ORIG) && kb == qb;   // the diagonal block; other own-segment blocks lie before it
+  // the first item's list, then its first tile
+  stage_list_async(list_row(a0, cur), a0->cap >> 3, LDS_LIST, wave, (int)threadIdx.x);
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  __syncthreads();
+  uint32_t li = 0;        // which list buffer holds the current item's list
+  uint32_t par = 0;       // which tile buffers hold the current item's first tile (0 or 0x8000)
+  {
+    stage_entry(head_base(a0, cur / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)reinterpret_cast<const uint16_t*>(smem + LDS_LIST)[1]), 0u,
+                (int)threadIdx.x & 63, async_lane_offset(wave, (int)threadIdx.x & 63));
+  }
 
-      // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
-      // single key yet (its reference maximum is still -inf)
-      if (first && !masked && !careful_only) {
-        // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good
-        // enough reference to start the pipelined path (later keys move it up lazily)
-        first = false;
-        f32x16 s0 = (f32x16){0};
+  bool careful_only = false;   // the current pass repeats an item without speculation
+  for (;;) {
+    const uint16_t* mlist = reinterpret_cast<const uint16_t*>(smem + LDS_LIST + li * LIST_BYTES);
+    const uint16_t* nlist = reinterpret_cast<const uint16_t*>(smem + LDS_LIST + (li ^ 1u) * LIST_BYTES);
+    ArgsPtr ap = PBS_ARGS();
+    // everything per lane is derived afresh from the lane id in every item: nothing but scalars lives across items
+    const int lane = lane_id_here();
+    const int tid = wave * 64 + lane;
+    const int j = lane & 31, gh = lane >> 5;
+    // per-lane LDS byte offsets of the fragments inside buffer 0; XOR 0x8000 switches buffer.
+    //   K fragment (sub-tile ks, d-step t)      : koff[t] + ks * 8192
+    //   V fragment (keys 16 c .. 16 c + 15, dt) : voff[c] + dt * 8192
+    // The 16-byte chunk index is XORed with the row: fragment t of a row lies at (offset of fragment 0) ^ (t << 5),
+    // so one per-lane offset per operand serves all eight; the XOR constant is merged with the buffer switch in
+    // scalar registers (bx[] below), one vector XOR per read either way.
+    const int krow = mfma_row_to_key(j);
+    const uint32_t koff0 = (uint32_t)(krow * 256 + ((gh ^ (krow & 15)) * 16));
+    const uint32_t voff0 = LDS_V0 + (uint32_t)(j * 256 + ((gh ^ (j & 15)) * 16));
+    const uint32_t lane_off = async_lane_offset(wave, lane);
+    int claim = 0;   // ticket of the next item: in flight during one tile
+
+    const int bh = cur / npair;
+    const int pair = npair - 1 - cur % npair;
+    const HeadBase hb = head_base(ap, bh);
+    const int b = bh / ap->Hq, h = bh % ap->Hq;
+    const int qb = 2 * pair + grp;
+    const bool qb_valid = qb < ap->nb;
+    const float c_log2 = ap->scale_log2;
+    const int qpos = qb * BS + 32 * wq + j;
+
+    // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7.  Rows past the end of the sequence
+    // compute on the last row's values and are never stored.
+    bf16x8 qf[8];
+    {
+      const uint16_t* qrow = ap->q + b * ap->q_sb + h * ap->q_sh + (int64_t)min(qpos, ap->S - 1) * ap->q_ss;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) s0 = PBS_MFMA(ldsf(koff[t] ^ bufx), qf[t], s0);
-        float mx = s0[0];
+      for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(qrow + 16 * t + 8 * gh);
+    }
+    const int n_tiles = __builtin_amdgcn_readfirstlane((int)mlist[0]);
+    // the next item: claimed three tiles before the end of this one (the counter's latency passes under a
+    // tile), published and its list and queries requested one tile later, its first tile requested at the last
+    // tile.  Items of fewer than three tiles finish these steps after their loop.
+    const int claim_it = careful_only ? -8 : max(n_tiles - 3, 0);
+    auto publish_and_fetch = [&]() {   // between the wait for this thread's loads and the barrier ...
+      if (wave == 0 && lane_id_here() == 0) misc[4] = q_begin + claim;
+    };
+    auto adopt_next = [&]() {          // ... and after the barrier
+      nxt = __builtin_amdgcn_readfirstlane(misc[4]);
+      has_nxt = nxt < q_end;
+      if (has_nxt) {
+        ArgsPtr an = PBS_ARGS();
+        const int ln = lane_id_here();
+        stage_list_async(list_row(an, nxt), an->cap >> 3, LDS_LIST + (li ^ 1u) * LIST_BYTES, wave, wave * 64 + ln);
+        // the next item's queries are read once, from HBM: bring this wave's 32 rows into L2 now (copies into a
+        // landing area nobody reads), so that the loads at the top of the item find them there
+        const int bh_n = nxt / npair, qb_n = 2 * (npair - 1 - nxt % npair) + grp;
+        const int pos0 = qb_n * BS + 32 * wq;
+        if (pos0 + 32 <= an->S) {
+          const int64_t q_ss = an->q_ss;
+          const uint16_t* qn = an->q + (bh_n / an->Hq) * an->q_sb + (bh_n % an->Hq) * an->q_sh + (int64_t)pos0 * q_ss;
+          const uint32_t voff = (uint32_t)((ln >> 4) * (uint32_t)q_ss * 2u + (ln & 15) * 16u);
 #pragma unroll
-        for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
-        mx = fmaxf(mx, xhalf_f32(mx));
-        m_ref = mx * c_log2;
-        all_seen = true;
-        fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
-      } else if (first || careful_only || (masked && !all_seen)) {
-        // ---------------- careful tile
-        first = false;
-        f32x16 s[4];
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
-          s[ks] = (f32x16){0};
-#pragma unroll
-          for (int t = 0; t < 8; ++t) s[ks] = PBS_MFMA(ldsf((koff[t] ^ bufx) + ks * 8192), qf[t], s[ks]);
+          for (int n = 0; n < 8; ++n) {
+            const uint64_t base = (uint64_t)(uintptr_t)(qn + 4 * n * q_ss);
+            const uint32_t b_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)base);
+            const uint32_t b_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(base >> 32));
+            const uint64_t bu = ((uint64_t)b_hi << 32) | b_lo;
+            register uint32_t m0v asm("m0") = (uint32_t)__builtin_amdgcn_readfirstlane((int)(LDS_DUMP + wave * 1024));
+            asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(bu) : "memory");
+          }
         }
-        if (masked) {
-          int qrel = 32 * wq + j;
-          asm volatile("" : "+v"(qrel));   // keep the compares inside the tile (see fast_tile)
+      }
+    };
+
+    {
+      f32x16 o[4];
+      {
+        float zero = 0.f;   // opaque: a constant zero vector would be kept (and spilled) as sixteen registers
+        asm volatile("" : "+v"(zero));
+#pragma unroll
+        for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) o[dt][r] = zero;
+      }
+      float m_ref = -INFINITY;   // reference maximum, identical in lanes j and j + 32
+      float l_part = 0.f;        // row sum of this lane's half of the keys
+      bool first = true, poisoned = false;
+      bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
+
+      if (careful_only) {
+        // the redo pass starts the item over: its first tile goes back into the buffers it had (the next
+        // item's first tile, if it was on its way there, is fetched again at the end of this pass)
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1]), par, lane, lane_off);
+      }
+      uint32_t bufx = par;
+      for (int it = 0; it < n_tiles; ++it, bufx ^= 0x8000u) {
+        const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
+        const int kb = (int)(ent & ENT_KB);
+        __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` (and of the next list) has landed
+        if (it == claim_it + 1) publish_and_fetch();
+        __syncthreads();                      // every share has; every wave is done with tile it - 1
+        if (it == claim_it + 1) adopt_next();
+        if (it == claim_it && wave == 0 && lane_id_here() == 0) claim = atomicAdd(PBS_ARGS()->queue + vic, 1);
+        if (it + 1 < n_tiles) stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
+        else if (has_nxt && (careful_only || n_tiles >= 3))   // shorter items: after the loop, once the list has landed
+          stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx ^ 0x8000u, lane, lane_off);
+        if (!(ent & use_bit) || !qb_valid) continue;
+        uint32_t bx[8];   // buffer switch ^ fragment index << 5: opaque, or the compiler folds the constant into eight per-lane offsets
+#pragma unroll
+        for (int t = 0; t < 8; ++t) {
+          bx[t] = bufx ^ (uint32_t)(t << 5);
+          asm volatile("" : "+s"(bx[t]));
+        }
+        const bool masked = (ent & ENT_ORIG) && kb == qb;   // the diagonal block; other own-segment blocks lie before it
+
+        // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
+        // single key yet (its reference maximum is still -inf)
+        if (first && !masked && !careful_only) {
+          // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good
+          // enough reference to start the pipelined path (later keys move it up lazily)
+          first = false;
+          f32x16 s0 = (f32x16){0};
+#pragma unroll
+          for (int t = 0; t < 8; ++t) s0 = PBS_MFMA(ldsf(koff0 ^ bx[t]), qf[t], s0);
+          float mx = s0[0];
+#pragma unroll
+          for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
+          mx = fmaxf(mx, xhalf_f32(mx));
+          m_ref = mx * c_log2;
+          all_seen = true;
+          fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
+        } else if (first || careful_only || (masked && !all_seen)) {
+          // ---------------- careful tile
+          first = false;
+          f32x16 s[4];
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks) {
+            s[ks] = (f32x16){0};
+#pragma unroll
+            for (int t = 0; t < 8; ++t) s[ks] = PBS_MFMA(ldsf((koff0 ^ bx[t]) + ks * 8192), qf[t], s[ks]);
+          }
+          if (masked) {
+            const int ln = lane_id_here();   // keep the compares inside the tile (see fast_tile)
+            const int qrel = 32 * wq + (ln & 31), gh = ln >> 5;
+#pragma unroll
+            for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int a4 = r >> 2;
+                const int key = 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1) + (r & 3);
+                if (key > qrel) s[ks][r] = -INFINITY;
+              }
+          }
+          float mx = -INFINITY;
+#pragma unroll
+          for (int ks = 0; ks < 4; ++ks)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[ks][r]);
+          mx = fmaxf(mx, xhalf_f32(mx));
+          const float m_new = fmaxf(m_ref, mx * c_log2);
+          const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+          const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
+          float rs = 0.f;
 #pragma unroll
           for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-              const int a4 = r >> 2;
-              const int key = 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1) + (r & 3);
-              if (key > qrel) s[ks][r] = -INFINITY;
+              const float p = __builtin_amdgcn_exp2f(s[ks][r] * c_log2 - m_use);
+              s[ks][r] = p;
+              rs += p;
             }
-        }
-        float mx = -INFINITY;
+          l_part = l_part * alpha + rs;
+          m_ref = m_new;
+          all_seen = !__any(m_ref == -INFINITY);
+          if (__any(alpha != 1.0f)) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
+            for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[ks][r]);
-        mx = fmaxf(mx, xhalf_f32(mx));
-        const float m_new = fmaxf(m_ref, mx * c_log2);
-        const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-        const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
-        float rs = 0.f;
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const float p = __builtin_amdgcn_exp2f(s[ks][r] * c_log2 - m_use);
-            s[ks][r] = p;
-            rs += p;
+              for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
           }
-        l_part = l_part * alpha + rs;
-        m_ref = m_new;
-        all_seen = !__any(m_ref == -INFINITY);
-        if (__any(alpha != 1.0f)) {
 #pragma unroll
-          for (int dt = 0; dt < 4; ++dt)
+          for (int ks = 0; ks < 4; ++ks)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+            for (int u = 0; u < 2; ++u) {
+              bf16x8 pf;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s[ks][8 * u + e];
+#pragma unroll
+              for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff0 ^ bx[2 * ks + u]) + dt * 8192), pf, o[dt]);
+            }
+        } else {
+          if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
+          else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
         }
-#pragma unroll
-        for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-          for (int u = 0; u < 2; ++u) {
-            bf16x8 pf;
-#pragma unroll
-            for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s[ks][8 * u + e];
-#pragma unroll
-            for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff[2 * ks + u] ^ bufx) + dt * 8192), pf, o[dt]);
-          }
-      } else {
-        if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
-        else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff, voff, bufx, c_log2, m_ref, l_part, poisoned, wq, j, gh);
       }
-    }
-    if (poisoned) misc[1] = 1;
-    __syncthreads();
-    if (!careful_only && misc[1] != 0) continue;   // the whole workgroup redoes both rows without speculation
+      if (!careful_only && n_tiles < 3) {
+        if (n_tiles < 2) {
+          __builtin_amdgcn_s_waitcnt(0x0f70);
+          publish_and_fetch();
+          __syncthreads();
+          adopt_next();
+        }
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        if (has_nxt)
+          stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx, lane, lane_off);
+      }
+      if (poisoned) misc[1] = 1;
+      __syncthreads();   // every wave is done with the last tile
+      if (!careful_only && misc[1] != 0) {   // the whole workgroup redoes both rows without speculation
+        careful_only = true;
+        continue;
+      }
 
-    // ---- epilogue: normalise, transpose through LDS (same swizzle), coalesced 16-byte stores
-    const float inv = 1.0f / (l_part + xhalf_f32(l_part));
-    uint16_t* os = reinterpret_cast<uint16_t*>(smem) + grp * (BS * D);
+      // ---- epilogue: normalise, transpose through LDS (same swizzle), coalesced 16-byte stores.  The staging
+      // area is the pair of buffers the last tile sat in (the other pair is receiving the next item's first
+      // tile): its K buffer for the first query block, its V buffer for the second.
+      const float inv = 1.0f / (l_part + xhalf_f32(l_part));
+      // lane-dependent addresses of the epilogue come from a fresh opaque lane id: derived from the item's one
+      // they would be computed at the top of the item and held across the tile loop
+      const int lane_e = lane_id_here();
+      const int j_e = lane_e & 31, gh_e = lane_e >> 5;
+      const uint32_t last_buf = par ^ (((n_tiles - 1) & 1) ? 0x8000u : 0u);
+      uint16_t* os = reinterpret_cast<uint16_t*>(smem + last_buf + (grp ? LDS_V0 : 0u));
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < 4; ++dt)
 #pragma unroll
-      for (int a4 = 0; a4 < 4; ++a4) {
-        const int row = 32 * wq + j;
-        const int c = 4 * dt + a4;   // 16-byte chunk of d = 32 dt + 8 a4 + 4 gh + 0..3
-        bf16x4 v4;
+        for (int a4 = 0; a4 < 4; ++a4) {
+          const int row = 32 * wq + j_e;
+          const int c = 4 * dt + a4;   // 16-byte chunk of d = 32 dt + 8 a4 + 4 gh + 0..3
+          bf16x4 v4;
 #pragma unroll
-        for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][4 * a4 + cc] * inv);
-        *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * gh) = v4;
-      }
-    __syncthreads();
-    if (qb_valid) {
-      uint16_t* obase = a.o + b * a.o_sb + h * a.o_sh;
-      // the query block index is rebuilt from the thread id here: keeping it alive across the tile loop
-      // costs a register the loop does not have
-      int tid_e = threadIdx.x;
-      asm volatile("" : "+v"(tid_e));
-      const int qb_e = 2 * pair + (tid_e >> 8);
-      const int t256 = tid_e & 255;
+          for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][4 * a4 + cc] * inv);
+          *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * gh_e) = v4;
+        }
+      __syncthreads();
+      if (qb_valid) {
+        ArgsPtr ae = PBS_ARGS();
+        const int bh_e = cur / npair;
+        uint16_t* obase = ae->o + (bh_e / ae->Hq) * ae->o_sb + (bh_e % ae->Hq) * ae->o_sh;
+        const int S_e = ae->S;
+        const int64_t o_ss = ae->o_ss;
+        // the query block index is rebuilt from the thread id here: keeping it alive across the tile loop
+        // costs a register the loop does not have
+        const int tid_e = wave * 64 + lane_e;
+        const int qb_e = 2 * (npair - 1 - cur % npair) + (tid_e >> 8);
+        const int t256 = tid_e & 255;
+        const uint16_t* os_e = reinterpret_cast<const uint16_t*>(smem + last_buf + ((tid_e >> 8) ? LDS_V0 : 0u));
 #pragma unroll
-      for (int n = 0; n < 8; ++n) {
-        const int ci = t256 + 256 * n;
-        const int row = ci >> 4, c = ci & 15;
-        const int pos = qb_e * BS + row;
-        if (pos < a.S)
-          *reinterpret_cast<u32x4*>(obase + (int64_t)pos * a.o_ss + c * 8) =
-              *reinterpret_cast<const u32x4*>(os + row * D + ((c ^ (row & 15)) * 8));
+        for (int n = 0; n < 8; ++n) {
+          const int ci = t256 + 256 * n;
+          const int row = ci >> 4, c = ci & 15;
+          const int pos = qb_e * BS + row;
+          if (pos < S_e)
+            *reinterpret_cast<u32x4*>(obase + (int64_t)pos * o_ss + c * 8) =
+                *reinterpret_cast<const u32x4*>(os_e + row * D + ((c ^ (row & 15)) * 8));
+        }
       }
     }
-    break;
+    if (!has_nxt) {
+      // the range is used up: serve the other XCDs' ranges, one after the other.  No look-ahead on this path:
+      // claim, fetch the list, request the first tile, each after the other
+      ArgsPtr as = PBS_ARGS();
+      while (vic_tried < 7) {
+        ++vic_tried;
+        vic = (xcd + vic_tried) & 7;
+        q_begin = as->xcd_start[vic];
+        q_end = as->xcd_start[vic + 1];
+        __syncthreads();   // everyone has read the previous ticket
+        if (wave == 0 && lane_id_here() == 0) misc[4] = q_begin + atomicAdd(as->queue + vic, 1);
+        __syncthreads();
+        nxt = __builtin_amdgcn_readfirstlane(misc[4]);
+        if (nxt < q_end) {
+          has_nxt = true;
+          break;
+        }
+      }
+      if (has_nxt) {
+        stage_list_async(list_row(as, nxt), as->cap >> 3, LDS_LIST + (li ^ 1u) * LIST_BYTES, wave, wave * 64 + lane_id_here());
+        __builtin_amdgcn_s_waitcnt(0x0f70);
+        __syncthreads();
+        stage_entry(head_base(as, nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]),
+                    par ^ ((n_tiles & 1) ? 0x8000u : 0u), lane, lane_off);
+      }
+    }
+    if (!has_nxt) break;
+    careful_only = false;
+    par ^= (n_tiles & 1) ? 0x8000u : 0u;
+    li ^= 1u;
+    cur = nxt;
+    nxt = q_end;
+    has_nxt = false;
+    if (wave == 0 && lane_id_here() == 0) misc[1] = 0;   // read by everyone before the epilogue's barrier, set again only after the next item's barriers
   }
 }
 
 std::atomic<uint64_t> g_lds_reserved{0};   // bit d: the kernel's LDS size has been raised on device d
+std::atomic<int> g_cu_count[64];           // CUs of device d (0: not looked up yet)
 
 }  // namespace
+
+// entries per merged list row (a multiple of 8: rows stay 16-byte aligned): the count, at most nb blocks of
+// earlier segments, at most bps + 1 own-segment blocks
+static int list_cap(int nb, int bps) { return (1 + nb + std::min(bps, nb) + 1 + 7) / 8 * 8; }
+
+// workspace: 256 bytes of work counters, then one merged visit list per pair of query blocks
+
+extern "C" size_t pbs_sparse_attn_workspace_bytes(int B, int Hq, int S, int segment_size) {
+  const int64_t nb = (S + BS - 1) / BS, npair = (nb + 1) / 2, cap = list_cap((int)nb, segment_size / BS);
+  return 256 + (size_t)B * Hq * npair * cap * 2;
+}
 
 extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k,
                                    const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B,
                                    int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size, int64_t q_sb,
                                    int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb,
-                                   int64_t o_sh, int64_t o_ss, float softmax_scale, void* stream) {
+                                   int64_t o_sh, int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
   PBS_REQUIRE(q && perm_k && perm_vt && k && orig_vt && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
+  PBS_REQUIRE(workspace && ((uintptr_t)workspace % 256) == 0, "pbs_sparse_attn_fwd: workspace must be a 256-byte aligned device buffer of pbs_sparse_attn_workspace_bytes()");
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_sparse_attn_fwd: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
   PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_sparse_attn_fwd: bad shape");
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_sparse_attn_fwd: segment_size must be a multiple of block_size");
@@ -524,7 +745,7 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
   AttnArgs a;
   a.q = (const uint16_t*)q; a.pk = (const uint16_t*)perm_k; a.pvt = (const uint16_t*)perm_vt;
   a.k = (const uint16_t*)k; a.ovt = (const uint16_t*)orig_vt;
-  a.cols = csr_cols; a.cnt = csr_cnt; a.o = (uint16_t*)out;
+  a.o = (uint16_t*)out;
   a.BH = B * Hq; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS; a.bps = segment_size / block_size;
   a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = (uint32_t)k_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
   a.scale_log2 = softmax_scale * 1.4426950408889634f;
@@ -551,11 +772,22 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
     a.xcd_start[x] = (int)start;
     if (x > 0) max_items = std::max(max_items, a.xcd_start[x] - a.xcd_start[x - 1]);
   }
-  const int64_t n_wg = (int64_t)8 * max_items;
-  // the kernel's dynamic LDS size is raised once per device, not per call
+  a.cap = list_cap(a.nb, a.bps);
+  PBS_REQUIRE((uint32_t)a.cap * 2 <= LIST_BYTES, "pbs_sparse_attn_fwd: visit list too long");
+  a.queue = (int*)workspace;
+  a.plist = (const uint16_t*)((char*)workspace + 256);
+  // the kernel's dynamic LDS size is raised once per device, not per call; the CU count is looked up once too
   int dev = 0;
   hipError_t attr = hipGetDevice(&dev);
   const bool tracked = attr == hipSuccess && dev >= 0 && dev < 64;
+  int n_cu = tracked ? g_cu_count[dev].load(std::memory_order_relaxed) : 0;
+  if (n_cu <= 0) {
+    if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n_cu <= 0) n_cu = 256;
+    if (tracked) g_cu_count[dev].store(n_cu, std::memory_order_relaxed);
+  }
+  // one workgroup per CU (the kernel's LDS leaves room for one), a multiple of 8 so that every XCD gets its share;
+  // fewer when there are fewer items
+  const int64_t n_wg = std::min<int64_t>((int64_t)8 * max_items, (int64_t)(n_cu + 7) / 8 * 8);
   if (attr == hipSuccess && !(tracked && (g_lds_reserved.load(std::memory_order_acquire) >> dev & 1))) {
     attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
     if (attr == hipSuccess && tracked) g_lds_reserved.fetch_or(1ull << dev, std::memory_order_release);
@@ -564,6 +796,8 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
     pbs_set_error("pbs_sparse_attn_fwd: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
     return (int)attr;
   }
+  hipLaunchKernelGGL(merge_pair_lists_kernel, dim3((unsigned)(a.BH * npair)), dim3(512), 0, (hipStream_t)stream, csr_cols, csr_cnt,
+                     (uint16_t*)((char*)workspace + 256), a.queue, a.nb, a.bps, a.cap);
   hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(512), LDS_TOTAL, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_sparse_attn_fwd");
 }

@@ -12,7 +12,7 @@ __global__ void identity_indices_kernel(int32_t* idx, int S_pad, int64_t total) 
 }
 
 struct Layout {
-  size_t scores, score_ws, idx, perm_k, perm_vt, orig_vt, pooled_k, pooled_q, probs, cols, cnt, select_ws, total;
+  size_t scores, score_ws, idx, perm_k, perm_vt, orig_vt, pooled_k, pooled_q, probs, cols, cnt, select_ws, attn_ws, total;
 };
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -36,6 +36,7 @@ Layout make_layout(int B, int Hq, int Hkv, int S, int D, int block_size, int seg
   L.cols = take(rows * nb * nb * 4);
   L.cnt = take(rows * nb * 4);
   L.select_ws = take(pbs_select_blocks_workspace_bytes((int)rows));
+  L.attn_ws = take(pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size));
   L.total = off;
   return L;
 }
@@ -103,8 +104,8 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
   if ((rc = pbs_select_blocks((const float*)(w + L.probs), threshold_per_row, threshold, threshold_is_int_one,
                               force_select_first_block, (const int32_t*)(w + L.idx), rows, S, block_size, segment_size,
                               nullptr, nullptr, (int32_t*)(w + L.cols), (int32_t*)(w + L.cnt), w + L.select_ws,
-                              L.total - L.select_ws, stream))) return rc;
+                              L.attn_ws - L.select_ws, stream))) return rc;
   return pbs_sparse_attn_fwd(q, w + L.perm_k, w + L.perm_vt, k, w + L.orig_vt, (const int32_t*)(w + L.cols),
                              (const int32_t*)(w + L.cnt), out, B, Hq, Hkv, S, head_dim, block_size, segment_size, q_sb,
-                             q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, stream);
+                             q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, w + L.attn_ws, stream);
 }

@@ -187,10 +187,11 @@ def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_s
     assert k.shape == (B, Hkv, S, D) and orig_vt.shape == (B, Hkv, nb, D, BLOCK)
     assert csr_cols.is_contiguous() and csr_cnt.is_contiguous()
     assert csr_cols.shape == (B, Hq, nb, nb) and csr_cnt.shape == (B, Hq, nb)
+    ws = torch.empty(max(lib.pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size), 256), dtype=torch.uint8, device=q.device)
     _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols),
                                        _ptr(csr_cnt), _ptr(out), B, Hq, Hkv, S, D, BLOCK, segment_size,
                                        q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                                       out.stride(0), out.stride(1), out.stride(2), softmax_scale, _stream()),
+                                       out.stride(0), out.stride(1), out.stride(2), softmax_scale, _ptr(ws), _stream()),
                "pbs_sparse_attn_fwd")
     return out
 
