@@ -64,12 +64,23 @@ int pbs_segment_argsort(const float* scores, int32_t* key_indices, int rows, int
  * orig_vt (may be null): (B, Hkv, nb, 128, 128), the V blocks in ORIGINAL key order,
  * transposed the same way and zero past S -- the attention kernel reads a query
  * block's own segment un-permuted, where the causal mask is a plain triangle.
+ * pooled_k may be null (no pooling).  block_needed (may be null): (B*Hq, nb) bytes as written by
+ * pbs_select_blocks; permuted blocks whose byte is zero are skipped and their perm_k / perm_vt
+ * tiles left unwritten (the attention kernel reads only the blocks on some visit list).
  * Replaces pbs_attn/src/permute_states.py:59-69, pbs_attn/src/pbs.py:213-215,
  * the key padding of pbs.py:78-79 and the key pooling of pbs_attn/src/utils.py:24-29. */
 int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
                   void* pooled_k, void* orig_vt, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
                   int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
-                  void* stream);
+                  const uint8_t* block_needed, void* stream);
+
+/* pooled_k of pbs_gather_kv (the same bits) without gathering anything: the permuted key blocks are
+ * pooled straight from k through key_indices.  block_needed (may be null): (B*Hq, nb) bytes, cleared
+ * here, for pbs_select_blocks to set.  With this the permutation of pbs_attn/src/pbs.py:185-190 can be
+ * deferred until the selection (pbs.py:195-209) has said which permuted blocks are read at all. */
+int pbs_pool_k_permuted(const void* k, const int32_t* key_indices, void* pooled_k, uint8_t* block_needed, int B,
+                        int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb, int64_t k_sh,
+                        int64_t k_ss, int key_pool_max, void* stream);
 
 /* Query-block pooling (mean with divisor 128, or max; rows past S count as zero).
  * pooled_q: (B, Hq, nb, 128) bf16.  Replaces pbs_attn/src/pbs.py:67-71 and
@@ -97,12 +108,15 @@ int pbs_block_logits_softmax_causal(const void* pooled_q, const void* pooled_k, 
  * csr_cnt (rows, nb): the ascending key blocks of sel_mask that lie in segments
  * strictly before the query block's -- the permuted tiles the attention kernel
  * visits (it adds the causal part of the query block's own segment itself).
+ * block_needed (may be null): (rows, nb) bytes, cleared by the caller (pbs_pool_k_permuted does);
+ * the byte of every key block that appears on some query block's visit list is set to 1.
  * Replaces pbs_attn/src/utils.py:38-86 and pbs_attn/src/pbs.py:10-25,119-127,209. */
 size_t pbs_select_blocks_workspace_bytes(int rows);
 int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
                       int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices, int rows,
                       int S, int block_size, int segment_size, uint8_t* sel_mask, uint8_t* final_mask,
-                      int32_t* csr_cols, int32_t* csr_cnt, void* workspace, size_t workspace_bytes, void* stream);
+                      int32_t* csr_cols, int32_t* csr_cnt, uint8_t* block_needed, void* workspace,
+                      size_t workspace_bytes, void* stream);
 
 /* Block-sparse flash-attention forward.  Query block qb attends to the permuted K /
  * transposed V tiles listed in csr_cols (earlier segments, no element mask) and to

@@ -10,6 +10,12 @@
 //                                  produced by B*Hkv extra grid rows of the same launch
 // A 256-byte source row is read by 16 lanes x 16 bytes; K/V may be stored at
 // the KV-head count (query head h reads KV head h / G).
+// The same kernel runs in two reduced forms so that a caller can gather only what the attention will read:
+//   * pooling only (POOL_ONLY): pooled_k of every permuted block straight from K through the indices, nothing
+//     else read or written -- the block estimate needs no more -- and the per-block "needed" flags cleared;
+//   * filtered: the permuted blocks whose "needed" flag (set by the block selection for every block some query
+//     block visits) is zero are skipped; their perm_k / perm_vt tiles stay unwritten.
+// The pooled values of the two forms are the same bits: same loads, same order of additions.
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
@@ -27,17 +33,24 @@ struct GatherArgs {
   uint16_t* perm_vt;
   uint16_t* pooled_k;
   uint16_t* orig_vt;
+  uint8_t* needed;     // (B*Hq, nb) or null: filter (full form), cleared (pooling-only form)
   int B, Hq, Hkv, S, nb;
   int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
   int pool_max;
 };
 
+template <bool POOL_ONLY>
 __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
-  __shared__ uint16_t vt[BS * VT_PITCH];
+  __shared__ uint16_t vt[POOL_ONLY ? 2 : BS * VT_PITCH];
   __shared__ float pool[16][D];
   const int kb = blockIdx.x;
-  const bool orig = (int)blockIdx.y >= a.B * a.Hq;   // extra grid rows: V of a KV head in original order
+  const bool orig = !POOL_ONLY && (int)blockIdx.y >= a.B * a.Hq;   // extra grid rows: V of a KV head in original order
   const int bh = orig ? (int)blockIdx.y - a.B * a.Hq : (int)blockIdx.y;
+  if (POOL_ONLY) {
+    if (a.needed && threadIdx.x == 0) a.needed[(int64_t)bh * a.nb + kb] = 0;
+  } else if (!orig && a.needed && a.needed[(int64_t)bh * a.nb + kb] == 0) {
+    return;
+  }
   const int heads = orig ? a.Hkv : a.Hq;
   const int b = bh / heads, h = bh % heads, kvh = orig ? h : h / (a.Hq / a.Hkv);
   const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;  // row group, 16-byte chunk
@@ -58,9 +71,9 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
     if (pos < a.S) {
       const int src = orig ? pos : idx[i];
       if (!orig) kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
-      vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
+      if (!POOL_ONLY) vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
     }
-    if (!orig) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
+    if (!POOL_ONLY && !orig) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float lo = bf16_bits_to_f32(kv[e] & 0xffffu), hi = bf16_bits_to_f32(kv[e] >> 16);
@@ -72,20 +85,21 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
         acc[2 * e + 1] += hi;
       }
       // stage V row-major (4-byte stores: the padded pitch keeps them aligned)
-      *reinterpret_cast<uint32_t*>(&vt[i * VT_PITCH + c * 8 + 2 * e]) = vv[e];
+      if (!POOL_ONLY) *reinterpret_cast<uint32_t*>(&vt[i * VT_PITCH + c * 8 + 2 * e]) = vv[e];
     }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) pool[rg][c * 8 + e] = acc[e];
   __syncthreads();
 
-  if (threadIdx.x < D && !orig) {
+  if (threadIdx.x < D && !orig && a.pooled_k) {
     float s = pool[0][threadIdx.x];
     for (int r = 1; r < 16; ++r) s = a.pool_max ? fmaxf(s, pool[r][threadIdx.x]) : s + pool[r][threadIdx.x];
     if (!a.pool_max) s = s / (float)BS;
     a.pooled_k[((int64_t)bh * a.nb + kb) * D + threadIdx.x] = (uint16_t)f32_to_bf16_bits(s);
   }
 
+  if (POOL_ONLY) return;
   // transposed write-out: thread (d, key group of 8) -> 16 bytes of row d
   uint16_t* vdst = (orig ? a.orig_vt : a.perm_vt) + ((int64_t)bh * a.nb + kb) * D * BS;
 #pragma unroll
@@ -145,8 +159,8 @@ __global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t
 extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
                              void* pooled_k, void* orig_vt, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
                              int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
-                             void* stream) {
-  PBS_REQUIRE(k && v && key_indices && perm_k && perm_vt && pooled_k, "pbs_gather_kv: null tensor pointer");
+                             const uint8_t* block_needed, void* stream) {
+  PBS_REQUIRE(k && v && key_indices && perm_k && perm_vt, "pbs_gather_kv: null tensor pointer");
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_gather_kv: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
   PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_gather_kv: bad shape");
   PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_ss % 8 == 0,
@@ -157,12 +171,31 @@ extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_in
   a.k = (const uint16_t*)k; a.v = (const uint16_t*)v; a.idx = key_indices;
   a.perm_k = (uint16_t*)perm_k; a.perm_vt = (uint16_t*)perm_vt; a.pooled_k = (uint16_t*)pooled_k;
   a.orig_vt = (uint16_t*)orig_vt;
+  a.needed = const_cast<uint8_t*>(block_needed);
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss; a.v_sb = v_sb; a.v_sh = v_sh; a.v_ss = v_ss;
   a.pool_max = key_pool_max;
-  // orig_vt may be null: then only the permuted outputs are produced
-  hipLaunchKernelGGL(gather_kv_kernel, dim3(a.nb, B * Hq + (orig_vt ? B * Hkv : 0)), dim3(256), 0, (hipStream_t)stream, a);
+  // orig_vt may be null: then only the permuted outputs are produced; pooled_k may be null: no pooling
+  hipLaunchKernelGGL(gather_kv_kernel<false>, dim3(a.nb, B * Hq + (orig_vt ? B * Hkv : 0)), dim3(256), 0, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_gather_kv");
+}
+
+extern "C" int pbs_pool_k_permuted(const void* k, const int32_t* key_indices, void* pooled_k, uint8_t* block_needed, int B,
+                                   int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb, int64_t k_sh,
+                                   int64_t k_ss, int key_pool_max, void* stream) {
+  PBS_REQUIRE(k && key_indices && pooled_k, "pbs_pool_k_permuted: null tensor pointer");
+  PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_pool_k_permuted: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
+  PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_pool_k_permuted: bad shape");
+  PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && ((uintptr_t)k % 16) == 0,
+              "pbs_pool_k_permuted: rows must be 16-byte aligned");
+  PBS_REQUIRE(B * Hq <= 65535, "pbs_pool_k_permuted: too many heads");
+  GatherArgs a = {};
+  a.k = (const uint16_t*)k; a.idx = key_indices; a.pooled_k = (uint16_t*)pooled_k; a.needed = block_needed;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
+  a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
+  a.pool_max = key_pool_max;
+  hipLaunchKernelGGL(gather_kv_kernel<true>, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
+  return pbs_check_launch("pbs_pool_k_permuted");
 }
 
 extern "C" int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim, int block_size,

@@ -12,7 +12,7 @@ __global__ void identity_indices_kernel(int32_t* idx, int S_pad, int64_t total) 
 }
 
 struct Layout {
-  size_t scores, score_ws, idx, perm_k, perm_vt, orig_vt, pooled_k, pooled_q, probs, cols, cnt, select_ws, attn_ws, total;
+  size_t scores, score_ws, idx, perm_k, perm_vt, orig_vt, pooled_k, pooled_q, probs, cols, cnt, needed, select_ws, attn_ws, total;
 };
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -35,6 +35,7 @@ Layout make_layout(int B, int Hq, int Hkv, int S, int D, int block_size, int seg
   L.probs = take(rows * nb * nb * 4);
   L.cols = take(rows * nb * nb * 4);
   L.cnt = take(rows * nb * 4);
+  L.needed = take(rows * nb);
   L.select_ws = take(pbs_select_blocks_workspace_bytes((int)rows));
   L.attn_ws = take(pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size));
   L.total = off;
@@ -93,18 +94,28 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
                              q_ss, k_sb, k_sh, k_ss, w + L.score_ws, L.idx - L.score_ws, stream))) return rc;
     if ((rc = pbs_segment_argsort((const float*)(w + L.scores), (int32_t*)(w + L.idx), rows, S, s_pad, segment_size, stream))) return rc;
   }
-  if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, w + L.pooled_k, w + L.orig_vt, B, Hq, Hkv,
-                          S,
-                          head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, stream))) return rc;
-  if (!threshold_is_int_one) {
+  // With a real threshold the permuted K / V are gathered AFTER the selection, and only the blocks some query
+  // block visits: the estimate needs no more than the pooled permuted key blocks, which come straight from K.
+  // (Every candidate selected: everything is visited, one full gather.)
+  uint8_t* needed = threshold_is_int_one ? nullptr : w + L.needed;
+  if (threshold_is_int_one) {
+    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, w + L.orig_vt, B, Hq, Hkv,
+                            S, head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, nullptr, stream))) return rc;
+  } else {
+    if ((rc = pbs_pool_k_permuted(k, (const int32_t*)(w + L.idx), w + L.pooled_k, needed, B, Hq, Hkv, S, head_dim, block_size,
+                                  k_sb, k_sh, k_ss, key_pool_max, stream))) return rc;
     if ((rc = pbs_pool_q(q, w + L.pooled_q, B, Hq, S, head_dim, block_size, q_sb, q_sh, q_ss, query_pool_max, stream))) return rc;
     if ((rc = pbs_block_logits_softmax(w + L.pooled_q, w + L.pooled_k, (float*)(w + L.probs), rows, nb, head_dim,
                                        segment_size / block_size, stream))) return rc;
   }
   if ((rc = pbs_select_blocks((const float*)(w + L.probs), threshold_per_row, threshold, threshold_is_int_one,
                               force_select_first_block, (const int32_t*)(w + L.idx), rows, S, block_size, segment_size,
-                              nullptr, nullptr, (int32_t*)(w + L.cols), (int32_t*)(w + L.cnt), w + L.select_ws,
+                              nullptr, nullptr, (int32_t*)(w + L.cols), (int32_t*)(w + L.cnt), needed, w + L.select_ws,
                               L.attn_ws - L.select_ws, stream))) return rc;
+  if (!threshold_is_int_one) {
+    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, w + L.orig_vt, B, Hq, Hkv,
+                            S, head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, needed, stream))) return rc;
+  }
   return pbs_sparse_attn_fwd(q, w + L.perm_k, w + L.perm_vt, k, w + L.orig_vt, (const int32_t*)(w + L.cols),
                              (const int32_t*)(w + L.cnt), out, B, Hq, Hkv, S, head_dim, block_size, segment_size, q_sb,
                              q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, w + L.attn_ws, stream);

@@ -30,6 +30,7 @@ struct SelectArgs {
   uint8_t* final_mask;     // (rows, nb, nb) or null: sel | own segment
   int32_t* csr_cols;       // (rows, nb, nb) or null
   int32_t* csr_cnt;        // (rows, nb)
+  uint8_t* needed;         // (rows, nb) or null: set to 1 for every key block on some query block's visit list
 };
 
 // Block that holds original key 0.  A segment-wise permutation keeps it inside the first segment, so that
@@ -197,6 +198,10 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
     for (int kb = k0; kb < k1; ++kb) {
       if (flag[kb] && kb < seg_first) a.csr_cols[row_off + w++] = kb;
     }
+  }
+  if (a.needed) {
+    for (int kb = k0; kb < k1; ++kb)
+      if (flag[kb] && kb < seg_first) a.needed[(int64_t)row * nb + kb] = 1;   // every writer stores the same value
   }
   if (threadIdx.x == 255) a.csr_cnt[(int64_t)row * nb + qb] = s_scan[255];
 }
@@ -367,6 +372,7 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
     }
     const uint64_t ballot = __ballot(visit);
     if (visit && a.csr_cols) a.csr_cols[row_off + base + __popcll(ballot & ((1ull << lane) - 1ull))] = kb;
+    if (visit && a.needed) a.needed[(int64_t)row * nb + kb] = 1;   // every writer stores the same value
     base += __popcll(ballot);
   }
   if (lane == 0) a.csr_cnt[(int64_t)row * nb + qb] = base;
@@ -379,8 +385,8 @@ extern "C" size_t pbs_select_blocks_workspace_bytes(int rows) { return (size_t)r
 extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
                                  int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices,
                                  int rows, int S, int block_size, int segment_size, uint8_t* sel_mask,
-                                 uint8_t* final_mask, int32_t* csr_cols, int32_t* csr_cnt, void* workspace,
-                                 size_t workspace_bytes, void* stream) {
+                                 uint8_t* final_mask, int32_t* csr_cols, int32_t* csr_cnt, uint8_t* block_needed,
+                                 void* workspace, size_t workspace_bytes, void* stream) {
   PBS_REQUIRE(key_indices && csr_cnt, "pbs_select_blocks: null index / count pointer");
   PBS_REQUIRE(threshold_is_int_one || block_attn_scores, "pbs_select_blocks: null score pointer");
   PBS_REQUIRE(rows > 0 && rows <= 65535 && S > 0, "pbs_select_blocks: bad shape");
@@ -396,6 +402,7 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   a.idx = key_indices; a.first_blk = (int32_t*)workspace;
   a.nb = nb; a.bs = block_size; a.bps = bps; a.S = S; a.n_pow2 = next_pow2_int(nb);
   a.sel_mask = sel_mask; a.final_mask = final_mask; a.csr_cols = csr_cols; a.csr_cnt = csr_cnt;
+  a.needed = block_needed;
   hipStream_t st = (hipStream_t)stream;
   if (force_select_first_block)
     hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size,

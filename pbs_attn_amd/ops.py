@@ -87,9 +87,12 @@ def segment_argsort(scores, seq_len, segment_size, block_size=BLOCK):
     return idx
 
 
-def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False):
+def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False, block_needed=None, want_pooled=True):
     """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128), pooled_k (B, Hq, nb, D) and, with
-    ``want_orig_vt``, orig_vt (B, Hkv, nb, D, 128): the V blocks in original order, transposed."""
+    ``want_orig_vt``, orig_vt (B, Hkv, nb, D, 128): the V blocks in original order, transposed.
+    ``block_needed`` ((B, Hq, nb) uint8, from ``select_blocks(..., block_needed=...)``) restricts the gather to
+    the blocks whose byte is set: the other tiles of perm_k / perm_vt stay uninitialised.  ``want_pooled=False``
+    returns None for pooled_k."""
     _check_bf16_cuda(k, v)
     if key_pool_mode not in ("mean", "max"):
         raise ValueError(f"Invalid key_pool_mode: {key_pool_mode}")
@@ -101,15 +104,39 @@ def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False):
     assert idx.shape == (B, Hq, nb * BLOCK) and idx.dtype == torch.int32 and idx.is_contiguous()
     perm_k = torch.empty((B, Hq, nb * BLOCK, D), dtype=k.dtype, device=k.device)
     perm_vt = torch.empty((B, Hq, nb, D, BLOCK), dtype=k.dtype, device=k.device)
-    pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device)
+    pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device) if want_pooled else None
     orig_vt = torch.empty((B, Hkv, nb, D, BLOCK), dtype=k.dtype, device=k.device) if want_orig_vt else None
+    if block_needed is not None:
+        assert block_needed.shape == (B, Hq, nb) and block_needed.dtype == torch.uint8 and block_needed.is_contiguous()
     _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k), _ptr(orig_vt),
                                  B, Hq, Hkv, S, D, BLOCK, k.stride(0), k.stride(1), k.stride(2),
-                                 v.stride(0), v.stride(1), v.stride(2), int(key_pool_mode == "max"), _stream()),
+                                 v.stride(0), v.stride(1), v.stride(2), int(key_pool_mode == "max"),
+                                 _ptr(block_needed), _stream()),
                "pbs_gather_kv")
     if want_orig_vt:
         return perm_k, perm_vt, pooled_k, orig_vt
     return perm_k, perm_vt, pooled_k
+
+
+def pool_k_permuted(k, idx, num_q_heads, key_pool_mode="mean"):
+    """pooled_k of ``gather_kv`` (the same bits) without gathering: the permuted key blocks are pooled straight
+    from ``k`` through ``idx``.  Also returns a cleared (B, Hq, nb) uint8 tensor for ``select_blocks`` to mark
+    the key blocks that are visited at all."""
+    _check_bf16_cuda(k)
+    if key_pool_mode not in ("mean", "max"):
+        raise ValueError(f"Invalid key_pool_mode: {key_pool_mode}")
+    lib = _lib.load()
+    k = _rows16(k)
+    B, Hkv, S, D = k.shape
+    Hq = num_q_heads
+    nb = (S + BLOCK - 1) // BLOCK
+    assert idx.shape == (B, Hq, nb * BLOCK) and idx.dtype == torch.int32 and idx.is_contiguous()
+    pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device)
+    needed = torch.empty((B, Hq, nb), dtype=torch.uint8, device=k.device)
+    _lib.check(lib.pbs_pool_k_permuted(_ptr(k), _ptr(idx), _ptr(pooled_k), _ptr(needed), B, Hq, Hkv, S, D, BLOCK,
+                                       k.stride(0), k.stride(1), k.stride(2), int(key_pool_mode == "max"), _stream()),
+               "pbs_pool_k_permuted")
+    return pooled_k, needed
 
 
 def pool_q(q, query_pool_mode="mean"):
@@ -145,9 +172,10 @@ def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment, causal_candidat
 
 
 def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segment_size,
-                  force_select_first_block=True, want_masks=True, want_csr=True, rows_shape=None):
+                  force_select_first_block=True, want_masks=True, want_csr=True, rows_shape=None, block_needed=None):
     """Returns (sel_mask, final_mask, csr_cols, csr_cnt).  ``threshold`` may be a
-    python float, the python int 1 (all candidates) or a (B, H) tensor."""
+    python float, the python int 1 (all candidates) or a (B, H) tensor.  ``block_needed``: a cleared
+    (B, H, nb) uint8 tensor; the byte of every key block on some visit list is set."""
     lib = _lib.load()
     B, H = idx.shape[:2]
     dev = idx.device
@@ -162,9 +190,12 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     cols = torch.empty((B, H, nb, nb), dtype=torch.int32, device=dev) if want_csr else None
     cnt = torch.empty((B, H, nb), dtype=torch.int32, device=dev)
     ws = torch.empty(max(lib.pbs_select_blocks_workspace_bytes(B * H), 16), dtype=torch.uint8, device=dev)
+    if block_needed is not None:
+        assert block_needed.shape == (B, H, nb) and block_needed.dtype == torch.uint8 and block_needed.is_contiguous()
     _lib.check(lib.pbs_select_blocks(_ptr(P), _ptr(thr_rows), thr, int(is_int_one), int(bool(force_select_first_block)),
                                      _ptr(idx), B * H, seq_len, block_size, segment_size, _ptr(sel), _ptr(fin),
-                                     _ptr(cols), _ptr(cnt), _ptr(ws), ws.numel(), _stream()), "pbs_select_blocks")
+                                     _ptr(cols), _ptr(cnt), _ptr(block_needed), _ptr(ws), ws.numel(), _stream()),
+               "pbs_select_blocks")
     return sel, fin, cols, cnt
 
 

@@ -116,6 +116,33 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
     return dict(block_attn_scores=P, block_mask=sel, final_mask=fin, csr_cols=cols, csr_cnt=cnt)
 
 
+def _select_then_gather(query_states, key_states, value_states, block_size, segment_size, threshold,
+                        force_select_first_block, query_pool_mode, key_pool_mode):
+    B, Hq, S, _ = query_states.shape
+    s_pad = (S + block_size - 1) // block_size * block_size
+    nseg, rem = S // segment_size, S % segment_size
+    if nseg == 0 or (nseg == 1 and rem == 0):
+        idx = _identity_indices(B, Hq, s_pad, query_states.device)
+    else:
+        scores = ops.score_keys(query_states, key_states, block_size, segment_size)
+        _mark("score")
+        idx = ops.segment_argsort(scores, S, segment_size, block_size)
+        _mark("sort")
+    pooled_k, needed = ops.pool_k_permuted(key_states, idx, Hq, key_pool_mode)
+    _mark("pool_k")
+    pooled_q = ops.pool_q(query_states, query_pool_mode)
+    P = ops.block_logits_softmax(pooled_q, pooled_k, segment_size // block_size)
+    _mark("estimate")
+    _, _, cols, cnt = ops.select_blocks(P, threshold, idx, S, block_size, segment_size, force_select_first_block,
+                                        want_masks=False, block_needed=needed)
+    _mark("select")
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode, want_orig_vt=True,
+                                                block_needed=needed, want_pooled=False)
+    _mark("gather")
+    perm = PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, orig_vt)
+    return perm, dict(block_attn_scores=P, csr_cols=cols, csr_cnt=cnt, block_needed=needed)
+
+
 def permuted_block_sparse_attn_fwd(
     query_states: torch.Tensor,
     key_states: torch.Tensor,
@@ -156,9 +183,16 @@ def permuted_block_sparse_attn_fwd(
         segment_size = (q_len + block_size - 1) // block_size * block_size
         threshold = 1
 
-    perm = apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode)
-    sel = permuted_block_selection(query_states, perm, block_size, segment_size, threshold, causal,
-                                   force_select_first_block, query_pool_mode, key_pool_mode, want_masks=False)
+    if isinstance(threshold, int) and threshold == 1:
+        # every candidate is selected: no estimate, one full gather
+        perm = apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode)
+        sel = permuted_block_selection(query_states, perm, block_size, segment_size, threshold, causal,
+                                       force_select_first_block, query_pool_mode, key_pool_mode, want_masks=False)
+    else:
+        # the order of the single-call path: the estimate runs on key blocks pooled straight from K, and K / V
+        # are gathered after the selection, only the blocks some query block visits
+        perm, sel = _select_then_gather(query_states, key_states, value_states, block_size, segment_size, threshold,
+                                        force_select_first_block, query_pool_mode, key_pool_mode)
     out = perm.attention(query_states, sel["csr_cols"], sel["csr_cnt"], segment_size, 1.0 / math.sqrt(head_dim))
     _mark("sparse_attn")
     # queries are not permuted (pbs.py:191-193): un-permutation is the identity

@@ -540,3 +540,74 @@ def test_unpermute_scatter_and_identity(dev, B, H, S):
     ops.unpermute(o_perm, q_idx, out=buf)
     assert torch.equal(buf, ref)
     assert ops.unpermute(o_perm) is o_perm
+
+
+# ---------------------------------------------------------------------------- deferred, filtered gather
+@pytest.mark.parametrize("Hq,Hkv,S,seg,mode", [(4, 2, 1024, 256, "mean"), (4, 1, 1500, 512, "max"), (2, 2, 4096, 1024, "mean")])
+def test_pooled_permuted_keys_without_a_gather_are_the_same_bits(dev, Hq, Hkv, S, seg, mode):
+    """pool_k_permuted pools the permuted key blocks straight from K: the same bits as the gather's pooled_k."""
+    q, k, v = small_case(1, Hq, Hkv, S, seed=31)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    idx = ops.segment_argsort(ops.score_keys(qd, kd, 128, seg), S, seg, 128)
+    _, _, pooled_ref = ops.gather_kv(kd, vd, idx, Hq, mode)
+    pooled, needed = ops.pool_k_permuted(kd, idx, Hq, mode)
+    assert torch.equal(pooled, pooled_ref)
+    assert needed.shape == (1, Hq, (S + 127) // 128) and int(needed.sum()) == 0          # cleared for the selection
+
+
+@pytest.mark.parametrize("S,seg,thr,kind", [(4096, 256, 0.9, "uniform_heavy"), (4096, 1024, 0.5, "strong_heavy"),
+                                            (3000, 512, 0.8, "strong_uniform"), (2048, 256, 1, "uniform_heavy")])
+def test_selection_marks_the_visited_blocks_and_the_filtered_gather_moves_exactly_those(dev, S, seg, thr, kind):
+    """block_needed = the key blocks on some query block's visit list (the selected blocks of earlier segments);
+    the filtered gather writes those tiles with the bits of the full gather and leaves the others untouched."""
+    B, Hq, Hkv = 1, 4, 2
+    q, k, v = small_case(B, Hq, Hkv, S, kind=kind, seed=41)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    nb, bps = (S + 127) // 128, seg // 128
+    idx = ops.segment_argsort(ops.score_keys(qd, kd, 128, seg), S, seg, 128)
+    pooled_k, needed = ops.pool_k_permuted(kd, idx, Hq)
+    Pm = ops.block_logits_softmax(ops.pool_q(qd), pooled_k, bps)
+    sel, fin, cols, cnt = ops.select_blocks(Pm, thr, idx, S, 128, seg, True, block_needed=needed)
+    # from the masks: selected and in a strictly earlier segment than the query block
+    qb = torch.arange(nb, device=dev).view(nb, 1)
+    kb = torch.arange(nb, device=dev).view(1, nb)
+    earlier = kb < (qb // bps) * bps
+    want = (sel & earlier).any(dim=2).to(torch.uint8)
+    assert torch.equal(needed, want)
+    if isinstance(thr, float):
+        assert 0 < int(needed.sum()) < needed.numel()        # the cases are meant to filter something
+    full_k, full_vt, _, full_ovt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    part_k, part_vt, none_pooled, part_ovt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True, block_needed=needed,
+                                                            want_pooled=False)
+    assert none_pooled is None and torch.equal(part_ovt, full_ovt)
+    m = needed.bool()
+    assert torch.equal(part_k.view(B, Hq, nb, 128, 128)[m], full_k.view(B, Hq, nb, 128, 128)[m])
+    assert torch.equal(part_vt[m], full_vt[m])
+    # and the attention over the partly gathered tiles is the attention over the full ones, bit for bit
+    out_full = ops.sparse_attn_fwd(qd, full_k, full_vt, kd, full_ovt, cols, cnt, seg)
+    out_part = ops.sparse_attn_fwd(qd, part_k, part_vt, kd, part_ovt, cols, cnt, seg)
+    assert torch.equal(out_full, out_part)
+
+
+def test_filtered_gather_leaves_unneeded_tiles_alone(dev):
+    q, k, v = small_case(1, 2, 2, 1024, seed=43)
+    kd, vd = k.to(dev), v.to(dev)
+    idx = torch.arange(1024, dtype=torch.int32, device=dev).view(1, 1, -1).expand(1, 2, -1).contiguous()
+    needed = torch.zeros((1, 2, 8), dtype=torch.uint8, device=dev)
+    needed[0, 1, 3] = 1
+    lib_k, lib_vt, _ = ops.gather_kv(kd, vd, idx, 2)          # reference tiles
+    import pbs_attn_amd._lib as L
+    # run the filtered gather into buffers pre-filled with a marker
+    from pbs_attn_amd.ops import _ptr, _stream
+    pk = torch.full_like(lib_k, 7.0)
+    pvt = torch.full_like(lib_vt, 7.0)
+    lib = L.load()
+    L.check(lib.pbs_gather_kv(_ptr(kd), _ptr(vd), _ptr(idx), _ptr(pk), _ptr(pvt), None, None, 1, 2, 2, 1024, 128, 128,
+                              kd.stride(0), kd.stride(1), kd.stride(2), vd.stride(0), vd.stride(1), vd.stride(2), 0,
+                              _ptr(needed), _stream()), "pbs_gather_kv")
+    torch.cuda.synchronize()
+    pk5, ref5 = pk.view(1, 2, 8, 128, 128), lib_k.view(1, 2, 8, 128, 128)
+    assert torch.equal(pk5[0, 1, 3], ref5[0, 1, 3]) and torch.equal(pvt[0, 1, 3], lib_vt[0, 1, 3])
+    keep = torch.ones((1, 2, 8), dtype=torch.bool, device=dev)
+    keep[0, 1, 3] = False
+    assert bool((pk5[keep] == 7.0).all()) and bool((pvt[keep] == 7.0).all())
