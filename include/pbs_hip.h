@@ -108,13 +108,18 @@ int pbs_block_logits_softmax_causal(const void* pooled_q, const void* pooled_k, 
  * csr_cnt (rows, nb): the ascending key blocks of sel_mask that lie in segments
  * strictly before the query block's -- the permuted tiles the attention kernel
  * visits (it adds the causal part of the query block's own segment itself).
+ * candidate_rule says which entries of a row of block_attn_scores can be non-zero, so that only those are
+ * sorted: 0 = any (the whole row is sorted, as the reference does), 1 = key blocks of segments strictly
+ * before the query block's (rows written by pbs_block_logits_softmax), 2 = key blocks up to and including
+ * the query block (pbs_block_logits_softmax_causal).  Entries outside the rule must be exactly zero; the
+ * result is then the same as with rule 0.
  * block_needed (may be null): (rows, nb) bytes, cleared by the caller (pbs_pool_k_permuted does);
  * the byte of every key block that appears on some query block's visit list is set to 1.
  * Replaces pbs_attn/src/utils.py:38-86 and pbs_attn/src/pbs.py:10-25,119-127,209. */
 size_t pbs_select_blocks_workspace_bytes(int rows);
 int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
-                      int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices, int rows,
-                      int S, int block_size, int segment_size, uint8_t* sel_mask, uint8_t* final_mask,
+                      int threshold_is_int_one, int force_select_first_block, int candidate_rule,
+                      const int32_t* key_indices, int rows, int S, int block_size, int segment_size, uint8_t* sel_mask, uint8_t* final_mask,
                       int32_t* csr_cols, int32_t* csr_cnt, uint8_t* block_needed, void* workspace,
                       size_t workspace_bytes, void* stream);
 

@@ -109,7 +109,8 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
                                        segment_size / block_size, stream))) return rc;
   }
   if ((rc = pbs_select_blocks((const float*)(w + L.probs), threshold_per_row, threshold, threshold_is_int_one,
-                              force_select_first_block, (const int32_t*)(w + L.idx), rows, S, block_size, segment_size,
+                              force_select_first_block, /*candidate_rule=*/1, (const int32_t*)(w + L.idx), rows, S, block_size,
+                              segment_size,
                               nullptr, nullptr, (int32_t*)(w + L.cols), (int32_t*)(w + L.cnt), needed, w + L.select_ws,
                               L.attn_ws - L.select_ws, stream))) return rc;
   if (!threshold_is_int_one) {

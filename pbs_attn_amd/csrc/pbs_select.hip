@@ -31,6 +31,8 @@ struct SelectArgs {
   int32_t* csr_cols;       // (rows, nb, nb) or null
   int32_t* csr_cnt;        // (rows, nb)
   uint8_t* needed;         // (rows, nb) or null: set to 1 for every key block on some query block's visit list
+  int cand_rule;           // which entries of a row can be non-zero: 0 any, 1 kb < first block of qb's segment, 2 kb <= qb
+  int qb_lo, qb_hi;        // wave kernel: the query blocks this launch covers
 };
 
 // Block that holds original key 0.  A segment-wise permutation keeps it inside the first segment, so that
@@ -260,9 +262,10 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
   const int nb = a.nb;
   const int nb_pad = (nb + 15) & ~15;
   uint8_t* flag = smem_w + wave * nb_pad;
-  const int64_t rq = (int64_t)blockIdx.x * 4 + wave;   // (row, qb) flattened
+  const int64_t rq = (int64_t)blockIdx.x * 4 + wave;   // (row, qb - qb_lo) flattened
   if (rq >= total_rows) return;
-  const int row = (int)(rq / nb), qb = (int)(rq % nb);
+  const int nqb = a.qb_hi - a.qb_lo;
+  const int row = (int)(rq / nqb), qb = a.qb_lo + (int)(rq % nqb);
   const int seg_first = (qb / a.bps) * a.bps;
   const int seg_end = min(seg_first + a.bps, nb);
   const int64_t row_off = ((int64_t)row * nb + qb) * nb;
@@ -273,12 +276,15 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
     for (int kb = lane; kb < seg_first; kb += 64) flag[kb] = 1;
   } else {
     const float* p = a.P + row_off;
+    // entries that are zero by construction sort behind every candidate (ties keep index order) and add nothing
+    // to the running sum: the row is sorted up to its last candidate only (the launch is sized for that)
+    const int count = a.cand_rule == 1 ? seg_first : a.cand_rule == 2 ? min(qb + 1, nb) : nb;
     uint64_t k[NPL];
 #pragma unroll
     for (int r = 0; r < NPL; ++r) {
       const int i = lane * NPL + r;
       uint64_t key = ~0ull;
-      if (i < nb) {
+      if (i < count) {
         float v = p[i];
         if (v != v) v = 0.f;
         else if (v == INFINITY) v = FLT_MAX;
@@ -292,7 +298,7 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
     const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
     float v[NPL];
 #pragma unroll
-    for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < nb) ? desc_key_value(k[r]) : 0.f;
+    for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < count) ? desc_key_value(k[r]) : 0.f;
     // parallel float64 prefix
     double loc[NPL];
     double c = 0.0;
@@ -345,10 +351,12 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
         }
       }
     }
-    if (first >= nb) first = -1;   // never reached (padding ranks cannot qualify: they add zero)
+    if (first >= count) first = -1;   // never reached (padding ranks cannot qualify: they add zero)
 #pragma unroll
     for (int r = 0; r < NPL; ++r)
       if (lane * NPL + r <= first) flag[(uint32_t)k[r]] = 1;
+    // a row without candidates is all zeros: sorted whole, its first entry is block 0 and the running sum is 0
+    if (count == 0 && 0.0f >= thr && lane == 0) flag[0] = 1;
   }
   __builtin_amdgcn_wave_barrier();
   if (a.force_first && lane == 0) {
@@ -383,13 +391,14 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
 extern "C" size_t pbs_select_blocks_workspace_bytes(int rows) { return (size_t)rows * sizeof(int32_t); }
 
 extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per_row, float threshold,
-                                 int threshold_is_int_one, int force_select_first_block, const int32_t* key_indices,
-                                 int rows, int S, int block_size, int segment_size, uint8_t* sel_mask,
+                                 int threshold_is_int_one, int force_select_first_block, int candidate_rule,
+                                 const int32_t* key_indices, int rows, int S, int block_size, int segment_size, uint8_t* sel_mask,
                                  uint8_t* final_mask, int32_t* csr_cols, int32_t* csr_cnt, uint8_t* block_needed,
                                  void* workspace, size_t workspace_bytes, void* stream) {
   PBS_REQUIRE(key_indices && csr_cnt, "pbs_select_blocks: null index / count pointer");
   PBS_REQUIRE(threshold_is_int_one || block_attn_scores, "pbs_select_blocks: null score pointer");
   PBS_REQUIRE(rows > 0 && rows <= 65535 && S > 0, "pbs_select_blocks: bad shape");
+  PBS_REQUIRE(candidate_rule >= 0 && candidate_rule <= 2, "pbs_select_blocks: candidate_rule must be 0, 1 or 2");
   PBS_REQUIRE(block_size > 0 && block_size <= 256, "pbs_select_blocks: block_size %d outside (0, 256]", block_size);
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_select_blocks: segment_size must be a multiple of block_size");
   const int nb = (S + block_size - 1) / block_size;
@@ -403,18 +412,43 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
   a.nb = nb; a.bs = block_size; a.bps = bps; a.S = S; a.n_pow2 = next_pow2_int(nb);
   a.sel_mask = sel_mask; a.final_mask = final_mask; a.csr_cols = csr_cols; a.csr_cnt = csr_cnt;
   a.needed = block_needed;
+  a.cand_rule = candidate_rule; a.qb_lo = 0; a.qb_hi = nb;
   hipStream_t st = (hipStream_t)stream;
   if (force_select_first_block)
     hipLaunchKernelGGL(first_token_block_kernel, dim3(rows), dim3(1024), 0, st, key_indices, a.first_blk, nb * block_size, block_size,
                        min(segment_size, nb * block_size));
   if (nb <= 1024) {
-    // one wave per row, four rows per workgroup
-    const int total = rows * nb;
+    // one wave per row, four rows per workgroup.  The sort network is sized for the longest row of a launch;
+    // where the number of candidates grows with the query block, the rows are launched in groups of like length
     const size_t lds_w = (size_t)4 * ((nb + 15) & ~15);
-    const dim3 grid((unsigned)((total + 3) / 4));
-    if (nb <= 64) hipLaunchKernelGGL(select_blocks_wave_kernel<1>, grid, dim3(256), lds_w, st, a, total);
-    else if (nb <= 256) hipLaunchKernelGGL(select_blocks_wave_kernel<4>, grid, dim3(256), lds_w, st, a, total);
-    else hipLaunchKernelGGL(select_blocks_wave_kernel<16>, grid, dim3(256), lds_w, st, a, total);
+    auto launch = [&](int npl, int qb_lo, int qb_hi) {
+      SelectArgs g = a;
+      g.qb_lo = qb_lo; g.qb_hi = qb_hi;
+      const int total = rows * (qb_hi - qb_lo);
+      const dim3 grid((unsigned)((total + 3) / 4));
+      switch (npl) {
+        case 1: hipLaunchKernelGGL(select_blocks_wave_kernel<1>, grid, dim3(256), lds_w, st, g, total); break;
+        case 2: hipLaunchKernelGGL(select_blocks_wave_kernel<2>, grid, dim3(256), lds_w, st, g, total); break;
+        case 4: hipLaunchKernelGGL(select_blocks_wave_kernel<4>, grid, dim3(256), lds_w, st, g, total); break;
+        case 8: hipLaunchKernelGGL(select_blocks_wave_kernel<8>, grid, dim3(256), lds_w, st, g, total); break;
+        default: hipLaunchKernelGGL(select_blocks_wave_kernel<16>, grid, dim3(256), lds_w, st, g, total); break;
+      }
+    };
+    if (candidate_rule == 0 || threshold_is_int_one) {
+      launch(threshold_is_int_one || nb <= 64 ? 1 : nb <= 128 ? 2 : nb <= 256 ? 4 : nb <= 512 ? 8 : 16, 0, nb);
+    } else {
+      int qb_lo = 0;
+      for (int npl = 1; npl <= 16 && qb_lo < nb; npl *= 2) {
+        // query blocks whose candidate count fits 64 * npl sorted entries
+        const int64_t lim = 64 * npl;
+        int64_t hi = candidate_rule == 1 ? (lim / bps + 1) * (int64_t)bps : lim;
+        if (npl == 16 || hi > nb) hi = nb;
+        if (hi > qb_lo) {
+          launch(npl, qb_lo, (int)hi);
+          qb_lo = (int)hi;
+        }
+      }
+    }
     return pbs_check_launch("pbs_select_blocks");
   }
   const size_t lds = (size_t)a.n_pow2 * sizeof(uint64_t) + (size_t)((nb + 15) / 16) * 16;

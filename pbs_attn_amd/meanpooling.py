@@ -51,7 +51,7 @@ def MeanPooling_prefill(
     # one block per segment: the visit list holds the selected blocks before the diagonal, the diagonal
     # block (MeanPooling.py:54-58) is the attention kernel's own-segment tile
     sel, fin, cols, cnt = ops.select_blocks(scores, thr, idx, q_len, block_size, block_size,
-                                            force_select_first_block, want_masks=return_masks)
+                                            force_select_first_block, want_masks=return_masks, candidate_rule=2)
     out = ops.sparse_attn_fwd(query_states, perm_k, perm_vt, key_states, orig_vt, cols, cnt, block_size)
     if return_masks:
         return out, dict(block_attn_scores=scores, block_mask=fin, csr_cnt=cnt)

@@ -172,10 +172,13 @@ def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment, causal_candidat
 
 
 def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segment_size,
-                  force_select_first_block=True, want_masks=True, want_csr=True, rows_shape=None, block_needed=None):
+                  force_select_first_block=True, want_masks=True, want_csr=True, rows_shape=None, block_needed=None,
+                  candidate_rule=0):
     """Returns (sel_mask, final_mask, csr_cols, csr_cnt).  ``threshold`` may be a
     python float, the python int 1 (all candidates) or a (B, H) tensor.  ``block_needed``: a cleared
-    (B, H, nb) uint8 tensor; the byte of every key block on some visit list is set."""
+    (B, H, nb) uint8 tensor; the byte of every key block on some visit list is set.  ``candidate_rule``: 0 = the
+    whole row is sorted (any score tensor); 1 / 2 = the scores come from ``block_logits_softmax`` without / with
+    ``causal_candidates`` and are zero outside its candidates, so only those are sorted (same result)."""
     lib = _lib.load()
     B, H = idx.shape[:2]
     dev = idx.device
@@ -193,7 +196,7 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     if block_needed is not None:
         assert block_needed.shape == (B, H, nb) and block_needed.dtype == torch.uint8 and block_needed.is_contiguous()
     _lib.check(lib.pbs_select_blocks(_ptr(P), _ptr(thr_rows), thr, int(is_int_one), int(bool(force_select_first_block)),
-                                     _ptr(idx), B * H, seq_len, block_size, segment_size, _ptr(sel), _ptr(fin),
+                                     int(candidate_rule), _ptr(idx), B * H, seq_len, block_size, segment_size, _ptr(sel), _ptr(fin),
                                      _ptr(cols), _ptr(cnt), _ptr(block_needed), _ptr(ws), ws.numel(), _stream()),
                "pbs_select_blocks")
     return sel, fin, cols, cnt

@@ -106,12 +106,14 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
     S = query_states.shape[2]
     is_int_one = isinstance(threshold, int) and threshold == 1   # pbs.py:120 (True counts, as there)
     P = block_attn_scores
+    rule = 0   # scores handed in: any values, the whole row is sorted
     if P is None and (not is_int_one or want_masks):
         pooled_q = ops.pool_q(query_states, query_pool_mode)
         P = ops.block_logits_softmax(pooled_q, perm.pooled_k, segment_size // block_size)
+        rule = 1   # zero outside the blocks of earlier segments
         _mark("estimate")
     sel, fin, cols, cnt = ops.select_blocks(P, threshold, perm.key_indices, S, block_size, segment_size,
-                                            force_select_first_block, want_masks=want_masks)
+                                            force_select_first_block, want_masks=want_masks, candidate_rule=rule)
     _mark("select")
     return dict(block_attn_scores=P, block_mask=sel, final_mask=fin, csr_cols=cols, csr_cnt=cnt)
 
@@ -134,7 +136,7 @@ def _select_then_gather(query_states, key_states, value_states, block_size, segm
     P = ops.block_logits_softmax(pooled_q, pooled_k, segment_size // block_size)
     _mark("estimate")
     _, _, cols, cnt = ops.select_blocks(P, threshold, idx, S, block_size, segment_size, force_select_first_block,
-                                        want_masks=False, block_needed=needed)
+                                        want_masks=False, block_needed=needed, candidate_rule=1)
     _mark("select")
     perm_k, perm_vt, _, orig_vt = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode, want_orig_vt=True,
                                                 block_needed=needed, want_pooled=False)

@@ -163,6 +163,12 @@ def test_select_blocks_bit_exact(dev, nb, bps, thr, force_first):
             for qb in qbs:
                 want = [kb for kb in range(nb) if ref_sel[b, h, qb, kb] and qseg[kb] < qseg[qb]]
                 assert cols[b, h, qb, :cnt[b, h, qb]].tolist() == want
+    # told that the scores are zero outside the candidates, the kernel sorts only those: the same result
+    sel1, fin1, cols1, cnt1 = ops.select_blocks(Pm.to(dev), thr_dev, idx_pad.to(dev), S, 128, seg, force_first,
+                                                candidate_rule=1)
+    assert torch.equal(sel1.cpu(), ref_sel) and torch.equal(fin1.cpu(), ref_fin) and torch.equal(cnt1.cpu(), cnt)
+    live = torch.arange(nb).view(1, 1, 1, nb) < cnt.unsqueeze(-1)
+    assert torch.equal(cols1.cpu()[live], cols[live])
 
 
 def test_select_blocks_threshold_kinds_follow_the_reference(dev):
