@@ -199,6 +199,9 @@ __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8],
       if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff0 ^ bx[mt]) + mstep * 8192);
       if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff0 ^ bx[2 * (mstep - 2) + (mt >> 2)]) + (mt & 3) * 8192);
     }
+    // the reads go out before this slot's matrix instructions: left to the scheduler they sink behind them
+    // (their address is formed in the slot) and the fragments arrive a slot late
+    __builtin_amdgcn_sched_barrier(0);
     if (step <= 3) {
       const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
       sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
