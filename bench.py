@@ -438,6 +438,7 @@ def main():
         "stage_ms": res["stage_ms"],
         "ms_per_step_staged": res["ms_per_step_staged"],
         "hbm_gbs": res["hbm_gbs"],
+        "gathered_block_fraction": res["gathered_block_fraction"],
         "dense_sdpa_ms": res.get("dense_sdpa_ms"),
         "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
         "speedup_vs_dense_sdpa": res.get("speedup_vs_dense_sdpa"),
