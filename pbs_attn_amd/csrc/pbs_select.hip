@@ -293,9 +293,59 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
       }
       k[r] = key;
     }
+    const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
+
+    // Rows whose mass sits in a few blocks need no sort: the largest remaining entry is taken out of the row
+    // (smallest composite key: value descending, ties by index -- the order of the sort) and added to the
+    // sequential float64 sum until float32(sum) reaches the threshold: the reference's decision, term by term.
+    // Tried only when EXTRACT_MAX times the row's largest value can reach the threshold; a row that does not
+    // get there in EXTRACT_MAX steps is sorted whole like any other.
+    bool decided = false;
+    if (NPL > 1) {
+      constexpr int EXTRACT_MAX = 16;
+      uint64_t best = k[0];
+#pragma unroll
+      for (int r = 1; r < NPL; ++r) best = k[r] < best ? k[r] : best;
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) {
+        const uint64_t o = shfl_xor_u64(best, off);
+        best = o < best ? o : best;
+      }
+      if (best != ~0ull && (float)((double)desc_key_value(best) * EXTRACT_MAX) >= thr) {
+        uint64_t w[NPL];
+#pragma unroll
+        for (int r = 0; r < NPL; ++r) w[r] = k[r];
+        double cum = 0.0;
+        uint32_t my_idx = 0;
+        int taken = 0;
+        for (int it = 0; it < EXTRACT_MAX; ++it) {
+          if (it > 0) {
+            best = w[0];
+#pragma unroll
+            for (int r = 1; r < NPL; ++r) best = w[r] < best ? w[r] : best;
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1) {
+              const uint64_t o = shfl_xor_u64(best, off);
+              best = o < best ? o : best;
+            }
+            if (best == ~0ull) break;   // the row has no further entry: not reached, let the sort path say so
+          }
+          if (lane == it) my_idx = (uint32_t)best;
+#pragma unroll
+          for (int r = 0; r < NPL; ++r) w[r] = (w[r] == best) ? ~0ull : w[r];
+          cum += (double)desc_key_value(best);
+          taken = it + 1;
+          if ((float)cum >= thr) {
+            decided = true;
+            break;
+          }
+        }
+        if (decided && lane < taken) flag[my_idx] = 1;
+      }
+    }
+    if (!decided) {
     wave_bitonic_sort<NPL>(k, lane);
 
-    const float thr = a.thr_rows ? a.thr_rows[row] : a.thr;
     float v[NPL];
 #pragma unroll
     for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < count) ? desc_key_value(k[r]) : 0.f;
@@ -355,6 +405,7 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
 #pragma unroll
     for (int r = 0; r < NPL; ++r)
       if (lane * NPL + r <= first) flag[(uint32_t)k[r]] = 1;
+    }   // !decided
     // a row without candidates is all zeros: sorted whole, its first entry is block 0 and the running sum is 0
     if (count == 0 && 0.0f >= thr && lane == 0) flag[0] = 1;
   }

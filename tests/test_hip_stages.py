@@ -617,3 +617,49 @@ def test_filtered_gather_leaves_unneeded_tiles_alone(dev):
     keep = torch.ones((1, 2, 8), dtype=torch.bool, device=dev)
     keep[0, 1, 3] = False
     assert bool((pk5[keep] == 7.0).all()) and bool((pvt[keep] == 7.0).all())
+
+
+@pytest.mark.parametrize("nb,bps,thr", [(100, 4, 0.9), (300, 8, 0.5), (300, 1, 0.99), (600, 8, 0.9), (1024, 8, 0.9),
+                                        (1024, 8, "tensor"), (1024, 2, 0.999)])
+@pytest.mark.parametrize("rule", [0, 1])
+def test_select_blocks_rows_with_concentrated_mass(dev, nb, bps, thr, rule):
+    """Rows whose probability mass sits in a few blocks are decided without a sort (largest entry after largest
+    entry, sequential float64 sum).  Peaked rows with many exactly equal values (bf16-valued logits: ties go by
+    index), rows that reach the threshold with the 15th, 16th or 17th largest entry (the boundary of that path),
+    uniform rows (which fall back to the sort) and rows of one dominant block, against the oracle."""
+    B, H, S = 1, 2, nb * 128
+    g = torch.Generator().manual_seed(nb * 13 + bps)
+    cand, _ = O.candidate_masks(nb, bps)
+    logits = (torch.randn((B, H, nb, nb), generator=g) * 1.5).bfloat16().float()
+    kinds = torch.arange(nb) % 5
+    # 0: as drawn (diffuse); 1: a few blocks carry +10; 2: sixteen or seventeen equal leaders; 3: one dominant block
+    for qb in range(nb):
+        n = int(cand[qb].sum())
+        if n == 0:
+            continue
+        kd = int(kinds[qb])
+        if kd == 1:
+            pick = torch.randperm(n, generator=g)[:max(1, min(n, 6))]
+            logits[:, :, qb, pick] += 10.0
+        elif kd == 2:
+            m = min(n, 15 + (qb % 3))
+            logits[:, :, qb, :n] = -4.0
+            pick = torch.randperm(n, generator=g)[:m]
+            logits[:, :, qb, pick] = 8.0
+        elif kd == 3:
+            logits[:, :, qb, int(torch.randint(0, n, (1,), generator=g))] += 30.0
+        elif kd == 4:
+            logits[:, :, qb, :n] = 0.0        # exactly uniform: every value tied
+    Pm = torch.softmax(logits.masked_fill(~cand, float("-inf")), -1)
+    Pm = torch.nan_to_num(Pm, nan=0.0)
+    if thr == "tensor":
+        thr = torch.tensor([[0.6, 0.97]])
+    idx_pad = torch.arange(nb * 128).expand(B, H, -1).int().contiguous()
+    ref_sel, ref_fin = _oracle_selection(Pm, thr, idx_pad, nb, bps, True)
+    thr_dev = thr.to(dev) if isinstance(thr, torch.Tensor) else thr
+    sel, fin, cols, cnt = ops.select_blocks(Pm.to(dev), thr_dev, idx_pad.to(dev), S, 128, bps * 128, True,
+                                            candidate_rule=rule)
+    assert torch.equal(sel.cpu(), ref_sel)
+    assert torch.equal(fin.cpu(), ref_fin)
+    earlier = torch.arange(nb).view(1, nb) < ((torch.arange(nb) // bps) * bps).view(nb, 1)
+    assert torch.equal(cnt.cpu(), (ref_sel & earlier).sum(-1).int())
