@@ -233,22 +233,22 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     # selection and moves only the key blocks some query block visits (fraction f of all permuted blocks)
     e = 2
     f = 1.0
-    if "pool_k" in stages:
+    if "pool" in stages:
         _, sel2 = P._select_then_gather(q, k, v, bs, seg, thr, True, "mean", "mean")
         f = float(sel2["block_needed"].float().mean().item())
         del sel2
     res["gathered_block_fraction"] = f
     kv_once = B * Hkv * S * D * e                       # one of K, V at the KV heads
     score_b = kv_once + B * Hq * bs * D * e + B * Hq * S * 4
-    pool_k_b = kv_once + B * Hq * S * 4 + B * Hq * nb * D * e
+    pool_b = kv_once + B * Hq * S * 4 + 2 * B * Hq * nb * D * e + B * Hq * S * D * e    # K, indices, Q in; pooled out
     # reads: the K and V rows of the gathered blocks (each row counted once per KV head at most), their indices,
     # V again for the original-order transposed copy; writes: the gathered tiles and that copy
     gather_b = (2 * min(f * B * Hq, B * Hkv) * S * D * e + f * B * Hq * S * 4 + kv_once
                 + 2 * f * B * Hq * S * D * e + kv_once)
-    est_b = B * Hq * S * D * e + B * Hq * nb * nb * 4
+    est_b = (0 if "pool" in stages else B * Hq * S * D * e) + 2 * B * Hq * nb * D * e + B * Hq * nb * nb * 4
     res["hbm_gbs"] = {
         "score": score_b / (stages["score"] * 1e-3) / 1e9 if "score" in stages else None,
-        "pool_k": pool_k_b / (stages["pool_k"] * 1e-3) / 1e9 if "pool_k" in stages else None,
+        "pool": pool_b / (stages["pool"] * 1e-3) / 1e9 if "pool" in stages else None,
         "gather": gather_b / (stages["gather"] * 1e-3) / 1e9,
         "estimate": est_b / (stages["estimate"] * 1e-3) / 1e9 if "estimate" in stages else None,
     }
@@ -335,7 +335,7 @@ def run_report(torch, path, steps, warmup):
              ("cfg1", {"kind": "strong_heavy", "segment": 1024}), ("cfg2", {"kind": "strong_heavy"}),
              ("cfg2", {"kind": "strong_uniform"})]
     lines = ["| workload | generator | S | B x Hq/Hkv | segment | thr | density | MeanPooling density | MeanPooling ms | pass ms | "
-             "attn ms | attn TFLOP/s | % MFMA peak | dense SDPA ms | speed-up vs dense | score/sort/pool_k/estimate/select/gather ms |",
+             "attn ms | attn TFLOP/s | % MFMA peak | dense SDPA ms | speed-up vs dense | score/sort/pool/estimate/select/gather ms |",
              "|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|---|"]
     out = []
     for name, ov in runs:
@@ -350,7 +350,7 @@ def run_report(torch, path, steps, warmup):
             f"{st['sparse_attn']:.2f} | {res['effective_tflops_attn_kernel']:.0f} | "
             f"{100 * res['effective_tflops_attn_kernel'] / PEAK_BF16_TFLOPS:.1f} | "
             f"{res['dense_sdpa_ms']:.2f} | {res['dense_sdpa_ms'] / res['ms_per_step']:.2f} | "
-            f"{st.get('score', 0):.2f}/{st.get('sort', 0):.2f}/{st.get('pool_k', 0):.2f}/{st.get('estimate', 0):.2f}/"
+            f"{st.get('score', 0):.2f}/{st.get('sort', 0):.2f}/{st.get('pool', 0):.2f}/{st.get('estimate', 0):.2f}/"
             f"{st['select']:.2f}/{st['gather']:.2f} |")
         log(lines[-1])
         out.append(res)

@@ -82,6 +82,14 @@ int pbs_pool_k_permuted(const void* k, const int32_t* key_indices, void* pooled_
                         int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb, int64_t k_sh,
                         int64_t k_ss, int key_pool_max, void* stream);
 
+/* pbs_pool_q and pbs_pool_k_permuted in one launch (the same bits as the two calls): the two kinds of
+ * workgroup alternate in launch order, so the key pooling's scattered row reads and the query pooling's
+ * streaming reads run side by side. */
+int pbs_pool_blocks(const void* q, const void* k, const int32_t* key_indices, void* pooled_q, void* pooled_k,
+                    uint8_t* block_needed, int B, int Hq, int Hkv, int S, int head_dim, int block_size,
+                    int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                    int query_pool_max, int key_pool_max, void* stream);
+
 /* Query-block pooling (mean with divisor 128, or max; rows past S count as zero).
  * pooled_q: (B, Hq, nb, 128) bf16.  Replaces pbs_attn/src/pbs.py:67-71 and
  * pbs_attn/src/utils.py:18-23. */

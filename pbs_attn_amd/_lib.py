@@ -19,6 +19,7 @@ SIGNATURES = {
     "pbs_segment_argsort": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
     "pbs_gather_kv": (c_int, [_P] * 7 + [_I] * 6 + [_L] * 6 + [_I, _P, _P]),
     "pbs_pool_k_permuted": (c_int, [_P] * 4 + [_I] * 6 + [_L] * 3 + [_I, _P]),
+    "pbs_pool_blocks": (c_int, [_P] * 6 + [_I] * 6 + [_L] * 6 + [_I, _I, _P]),
     "pbs_pool_q": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P]),
     "pbs_block_logits_softmax": (c_int, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "pbs_block_logits_softmax_causal": (c_int, [_P, _P, _P, _I, _I, _I, _P]),

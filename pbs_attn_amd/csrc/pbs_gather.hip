@@ -40,12 +40,9 @@ struct GatherArgs {
 };
 
 template <bool POOL_ONLY>
-__global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
-  __shared__ uint16_t vt[POOL_ONLY ? 2 : BS * VT_PITCH];
-  __shared__ float pool[16][D];
-  const int kb = blockIdx.x;
-  const bool orig = !POOL_ONLY && (int)blockIdx.y >= a.B * a.Hq;   // extra grid rows: V of a KV head in original order
-  const int bh = orig ? (int)blockIdx.y - a.B * a.Hq : (int)blockIdx.y;
+__device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float (&pool)[16][D], int kb, int grid_row) {
+  const bool orig = !POOL_ONLY && grid_row >= a.B * a.Hq;   // extra grid rows: V of a KV head in original order
+  const int bh = orig ? grid_row - a.B * a.Hq : grid_row;
   if (POOL_ONLY) {
     if (a.needed && threadIdx.x == 0) a.needed[(int64_t)bh * a.nb + kb] = 0;
   } else if (!orig && a.needed && a.needed[(int64_t)bh * a.nb + kb] == 0) {
@@ -115,11 +112,17 @@ __global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
   }
 }
 
-// Mean / max pooling of Q blocks (rows past S count as zeros, the divisor stays 128).
-__global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t* pooled, int Hq, int S, int nb,
-                                                     int64_t q_sb, int64_t q_sh, int64_t q_ss, int pool_max) {
+template <bool POOL_ONLY>
+__global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
+  __shared__ uint16_t vt[POOL_ONLY ? 2 : BS * VT_PITCH];
   __shared__ float pool[16][D];
-  const int qb = blockIdx.x, bh = blockIdx.y;
+  gather_block<POOL_ONLY>(a, vt, pool, blockIdx.x, blockIdx.y);
+}
+
+
+// Mean / max pooling of Q blocks (rows past S count as zeros, the divisor stays 128).
+__device__ __forceinline__ void pool_q_block(float (&pool)[16][D], const uint16_t* q, uint16_t* pooled, int Hq, int S, int nb,
+                                             int64_t q_sb, int64_t q_sh, int64_t q_ss, int pool_max, int qb, int bh) {
   const int b = bh / Hq, h = bh % Hq;
   const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;
   const uint16_t* src = q + b * q_sb + h * q_sh;
@@ -152,6 +155,30 @@ __global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t
     if (!pool_max) s = s / (float)BS;
     pooled[((int64_t)bh * nb + qb) * D + threadIdx.x] = (uint16_t)f32_to_bf16_bits(s);
   }
+}
+
+__global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t* pooled, int Hq, int S, int nb,
+                                                     int64_t q_sb, int64_t q_sh, int64_t q_ss, int pool_max) {
+  __shared__ float pool[16][D];
+  pool_q_block(pool, q, pooled, Hq, S, nb, q_sb, q_sh, q_ss, pool_max, blockIdx.x, blockIdx.y);
+}
+
+// Both poolings of the block estimate in one launch, the two kinds of workgroup alternating in launch order: the
+// pooling of permuted key blocks waits on scattered 256-byte rows, the pooling of query blocks streams Q from
+// HBM; side by side each fills what the other leaves idle.
+struct PoolQArgs {
+  const uint16_t* q;
+  uint16_t* pooled_q;
+  int64_t q_sb, q_sh, q_ss;
+  int pool_max;
+};
+
+__global__ __launch_bounds__(256) void pool_qk_kernel(GatherArgs a, PoolQArgs p) {
+  __shared__ uint16_t vt[2];
+  __shared__ float pool[16][D];
+  const int bh = blockIdx.y >> 1;
+  if (blockIdx.y & 1) pool_q_block(pool, p.q, p.pooled_q, a.Hq, a.S, a.nb, p.q_sb, p.q_sh, p.q_ss, p.pool_max, blockIdx.x, bh);
+  else gather_block<true>(a, vt, pool, blockIdx.x, bh);
 }
 
 }  // namespace
@@ -196,6 +223,29 @@ extern "C" int pbs_pool_k_permuted(const void* k, const int32_t* key_indices, vo
   a.pool_max = key_pool_max;
   hipLaunchKernelGGL(gather_kv_kernel<true>, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_pool_k_permuted");
+}
+
+extern "C" int pbs_pool_blocks(const void* q, const void* k, const int32_t* key_indices, void* pooled_q, void* pooled_k,
+                               uint8_t* block_needed, int B, int Hq, int Hkv, int S, int head_dim, int block_size,
+                               int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss,
+                               int query_pool_max, int key_pool_max, void* stream) {
+  PBS_REQUIRE(q && k && key_indices && pooled_q && pooled_k, "pbs_pool_blocks: null tensor pointer");
+  PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_pool_blocks: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
+  PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_pool_blocks: bad shape");
+  PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 &&
+                  ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0,
+              "pbs_pool_blocks: rows must be 16-byte aligned");
+  PBS_REQUIRE(2 * B * Hq <= 65535, "pbs_pool_blocks: too many heads");
+  GatherArgs a = {};
+  a.k = (const uint16_t*)k; a.idx = key_indices; a.pooled_k = (uint16_t*)pooled_k; a.needed = block_needed;
+  a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
+  a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
+  a.pool_max = key_pool_max;
+  PoolQArgs p;
+  p.q = (const uint16_t*)q; p.pooled_q = (uint16_t*)pooled_q; p.q_sb = q_sb; p.q_sh = q_sh; p.q_ss = q_ss;
+  p.pool_max = query_pool_max;
+  hipLaunchKernelGGL(pool_qk_kernel, dim3(a.nb, 2 * B * Hq), dim3(256), 0, (hipStream_t)stream, a, p);
+  return pbs_check_launch("pbs_pool_blocks");
 }
 
 extern "C" int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim, int block_size,

@@ -102,9 +102,9 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
     if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, w + L.orig_vt, B, Hq, Hkv,
                             S, head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, nullptr, stream))) return rc;
   } else {
-    if ((rc = pbs_pool_k_permuted(k, (const int32_t*)(w + L.idx), w + L.pooled_k, needed, B, Hq, Hkv, S, head_dim, block_size,
-                                  k_sb, k_sh, k_ss, key_pool_max, stream))) return rc;
-    if ((rc = pbs_pool_q(q, w + L.pooled_q, B, Hq, S, head_dim, block_size, q_sb, q_sh, q_ss, query_pool_max, stream))) return rc;
+    if ((rc = pbs_pool_blocks(q, k, (const int32_t*)(w + L.idx), w + L.pooled_q, w + L.pooled_k, needed, B, Hq, Hkv, S,
+                              head_dim, block_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, query_pool_max, key_pool_max,
+                              stream))) return rc;
     if ((rc = pbs_block_logits_softmax(w + L.pooled_q, w + L.pooled_k, (float*)(w + L.probs), rows, nb, head_dim,
                                        segment_size / block_size, stream))) return rc;
   }

@@ -139,6 +139,28 @@ def pool_k_permuted(k, idx, num_q_heads, key_pool_mode="mean"):
     return pooled_k, needed
 
 
+def pool_blocks(q, k, idx, query_pool_mode="mean", key_pool_mode="mean"):
+    """``pool_q`` and ``pool_k_permuted`` in one launch: returns (pooled_q, pooled_k, block_needed)."""
+    _check_bf16_cuda(q, k)
+    for mode in (query_pool_mode, key_pool_mode):
+        if mode not in ("mean", "max"):
+            raise ValueError(f"Invalid pool mode: {mode}")
+    lib = _lib.load()
+    q, k = _rows16(q), _rows16(k)
+    B, Hq, S, D = q.shape
+    Hkv = k.shape[1]
+    nb = (S + BLOCK - 1) // BLOCK
+    assert idx.shape == (B, Hq, nb * BLOCK) and idx.dtype == torch.int32 and idx.is_contiguous()
+    pooled_q = torch.empty((B, Hq, nb, D), dtype=q.dtype, device=q.device)
+    pooled_k = torch.empty((B, Hq, nb, D), dtype=q.dtype, device=q.device)
+    needed = torch.empty((B, Hq, nb), dtype=torch.uint8, device=q.device)
+    _lib.check(lib.pbs_pool_blocks(_ptr(q), _ptr(k), _ptr(idx), _ptr(pooled_q), _ptr(pooled_k), _ptr(needed), B, Hq, Hkv,
+                                   S, D, BLOCK, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1),
+                                   k.stride(2), int(query_pool_mode == "max"), int(key_pool_mode == "max"), _stream()),
+               "pbs_pool_blocks")
+    return pooled_q, pooled_k, needed
+
+
 def pool_q(q, query_pool_mode="mean"):
     _check_bf16_cuda(q)
     if query_pool_mode not in ("mean", "max"):

@@ -130,9 +130,8 @@ def _select_then_gather(query_states, key_states, value_states, block_size, segm
         _mark("score")
         idx = ops.segment_argsort(scores, S, segment_size, block_size)
         _mark("sort")
-    pooled_k, needed = ops.pool_k_permuted(key_states, idx, Hq, key_pool_mode)
-    _mark("pool_k")
-    pooled_q = ops.pool_q(query_states, query_pool_mode)
+    pooled_q, pooled_k, needed = ops.pool_blocks(query_states, key_states, idx, query_pool_mode, key_pool_mode)
+    _mark("pool")
     P = ops.block_logits_softmax(pooled_q, pooled_k, segment_size // block_size)
     _mark("estimate")
     _, _, cols, cnt = ops.select_blocks(P, threshold, idx, S, block_size, segment_size, force_select_first_block,

@@ -663,3 +663,15 @@ def test_select_blocks_rows_with_concentrated_mass(dev, nb, bps, thr, rule):
     assert torch.equal(fin.cpu(), ref_fin)
     earlier = torch.arange(nb).view(1, nb) < ((torch.arange(nb) // bps) * bps).view(nb, 1)
     assert torch.equal(cnt.cpu(), (ref_sel & earlier).sum(-1).int())
+
+
+@pytest.mark.parametrize("Hq,Hkv,S,seg,qmode,kmode", [(4, 2, 1024, 256, "mean", "mean"), (4, 1, 1500, 512, "max", "mean"),
+                                                      (6, 6, 2048, 1024, "mean", "max")])
+def test_both_poolings_in_one_launch_are_the_same_bits(dev, Hq, Hkv, S, seg, qmode, kmode):
+    q, k, v = small_case(2, Hq, Hkv, S, seed=51)
+    qd, kd = q.to(dev), k.to(dev)
+    idx = ops.segment_argsort(ops.score_keys(qd, kd, 128, seg), S, seg, 128)
+    pq, pk, needed = ops.pool_blocks(qd, kd, idx, qmode, kmode)
+    assert torch.equal(pq, ops.pool_q(qd, qmode))
+    assert torch.equal(pk, ops.pool_k_permuted(kd, idx, Hq, kmode)[0])
+    assert int(needed.sum()) == 0
