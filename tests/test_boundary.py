@@ -301,3 +301,22 @@ def test_ttft_model_specs_match_the_named_architectures():
         (4096, 32, 32, 8, 128, 14336, 128256, 500000.0)
     q = MODELS["qwen25_7b"]
     assert (q["num_attention_heads"], q["num_key_value_heads"], q["hidden_size"] // q["num_attention_heads"]) == (28, 4, 128)
+
+
+def test_operator_is_registered_with_the_dispatcher():
+    """torch.ops.pbs_hip.prefill_attn_fwd: schema, shape-only implementation for tracing, no CPU kernel."""
+    import pbs_attn_amd.torch_ops as T
+    schema = str(torch.ops.pbs_hip.prefill_attn_fwd.default._schema)
+    assert schema.startswith("pbs_hip::prefill_attn_fwd(Tensor q, Tensor k, Tensor v, int block_size, int segment_size")
+    assert "Tensor? threshold_per_head" in schema and schema.endswith("-> Tensor")
+    q = torch.empty(2, 4, 300, 128, dtype=torch.bfloat16, device="meta")
+    k = torch.empty(2, 2, 300, 128, dtype=torch.bfloat16, device="meta")
+    out = T.prefill_attn_fwd(q, k, k, 128, 256, 0.9)
+    assert out.shape == q.shape and out.dtype == q.dtype and out.device.type == "meta"
+    out = T.prefill_attn_fwd(q, k, k, 128, 256, torch.full((2, 4), 0.8, device="meta"))
+    assert out.shape == q.shape
+    with pytest.raises(RuntimeError):     # the shape checks of the tracing implementation
+        T.prefill_attn_fwd(q, k[:, :, :200], k[:, :, :200])
+    qc = torch.zeros(1, 2, 256, 128, dtype=torch.bfloat16)
+    with pytest.raises(NotImplementedError, match="CPU"):   # no CPU kernel, no fallback
+        T.prefill_attn_fwd(qc, qc, qc)

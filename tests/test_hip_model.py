@@ -66,3 +66,24 @@ def test_ttft_harness_defaults_follow_the_protocol():
     from pbs_attn_amd import ttft
     src = inspect.getsource(ttft.main)
     assert 'default=30, dest="num_warmup_iter"' in src and 'default=10, dest="n_examples"' in src
+
+
+def test_dispatcher_op_equals_the_direct_call_and_traces(dev):
+    """torch.ops.pbs_hip.prefill_attn_fwd gives the bits of the ctypes call, for the three threshold forms, and a
+    function that uses it can be captured by torch.compile's tracer (the op is one opaque node)."""
+    import pbs_attn_amd.torch_ops as T
+    from pbs_attn_amd import ops
+    from tests.util import small_case
+    q, k, v = small_case(2, 4, 2, 1500, seed=61)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    per_head = torch.tensor([[0.5, 0.7, 0.9, 0.95], [0.6, 0.8, 0.85, 0.99]], device=dev)
+    for thr in (0.9, 1, per_head):
+        direct = ops.prefill_attn_fwd(qd, kd, vd, 128, 256, thr)
+        via_op = T.prefill_attn_fwd(qd, kd, vd, 128, 256, thr)
+        assert torch.equal(direct, via_op)
+
+    def f(a, b, c):
+        return torch.ops.pbs_hip.prefill_attn_fwd(a * 1, b, c, 128, 256, 0.9, False, None, True, "mean", "mean") + 0
+
+    traced = torch.compile(f, backend="eager", fullgraph=True)
+    assert torch.equal(traced(qd, kd, vd), ops.prefill_attn_fwd(qd, kd, vd, 128, 256, 0.9))
