@@ -111,6 +111,43 @@ def mfma_ceiling(torch, iters=200000):
     return out
 
 
+def tile_pipeline(torch, iters=6000):
+    """The attention kernel's tile pipeline by itself (pbs_attn_tile_probe: fast tiles out of LDS with the
+    kernel's barrier and copies per tile, no lists, items or write-out), on all-zero and on normally distributed
+    K / V / Q: cycles per tile (the same on both), the time per tile and the shader clock the chip holds.  On data
+    the clock falls with the power limit; what the attention kernel reaches of this rate is the cost of
+    everything around the pipeline."""
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    dev = torch.device("cuda")
+    n_src = 256                                     # 16 MB ring of tile pairs
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    gen = torch.Generator(device="cpu").manual_seed(11)
+    rings = {"zeros": torch.zeros(n_src * 32768, dtype=torch.bfloat16, device=dev),
+             "normal": torch.randn(n_src * 32768, generator=gen).to(torch.bfloat16).to(dev)}
+    st = torch.cuda.current_stream().cuda_stream
+    out = {"kernel": "fast tiles of 128 keys x 256 queries per workgroup, 256 workgroups x 8 waves, barrier per tile",
+           "flop_per_tile_step": 2 * FLOP_PER_BLOCK_PAIR}
+    for name, ring in rings.items():
+        for copies in (1, 0):
+            clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+            args = (ring.data_ptr(), n_src, None, copies, sink.data_ptr(), clocks.data_ptr(), st)
+            _lib.check(lib.pbs_attn_tile_probe(*args[:2], iters // 8, *args[3:]), "pbs_attn_tile_probe")
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.pbs_attn_tile_probe(*args[:2], iters, *args[3:]), "pbs_attn_tile_probe")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            c = clocks.tolist()
+            key = name + ("" if copies else "_no_copies")
+            out[key] = {"us_per_tile_step": ms * 1e3 / iters, "cycles_per_tile_step": c[0] / iters,
+                        "shader_clock_mhz": 100.0 * c[0] / max(1, c[1]),
+                        "tflops": 256 * 2 * FLOP_PER_BLOCK_PAIR * iters / (ms * 1e-3) / 1e12}
+    return out
+
+
 def block_pair_counts(csr_cnt, B, Hq, nb, bps):
     """(executed, reference) numbers of 128 x 128 tiles of one launch.  executed = what the HIP kernel
     multiplies: the selected blocks of earlier segments plus the causal part of the own segment (blocks
@@ -449,6 +486,8 @@ def main():
         line["mfma_ceiling"] = mfma_ceiling(torch)
         line["roofline"]["frac_of_measured_ceiling"] = achieved / line["mfma_ceiling"]["normal"]
         line["roofline"]["kernel_ms_zero_operands"] = res["attn_ms_zero_operands"]
+        line["tile_pipeline"] = tile_pipeline(torch)
+        line["roofline"]["frac_of_tile_pipeline"] = achieved / line["tile_pipeline"]["normal"]["tflops"]
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(*inputs, seconds_budget=args.cpu_seconds)
     del inputs

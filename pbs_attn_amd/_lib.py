@@ -31,6 +31,7 @@ SIGNATURES = {
     "pbs_rope_qk": (c_int, [_P] * 6 + [_I] * 5 + [_L] * 8 + [_P]),
     "pbs_mfma_probe": (c_int, [_P, _I, _P, _P, _P]),
     "pbs_mfma_probe_flop": (ctypes.c_double, [_I]),
+    "pbs_attn_tile_probe": (c_int, [_P, _I, _I, _I, _P, _P, _P]),
     "pbs_identity_indices": (c_int, [_P, _I, _I, _P]),
     "pbs_prefill_attn_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I, _I]),
     "pbs_prefill_attn_fwd": (c_int, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 12 +

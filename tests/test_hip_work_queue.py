@@ -63,3 +63,20 @@ def test_work_distribution_shapes_against_dense_attention_on_the_mask(dev, B, Hq
     logits = qd.float() @ kf.transpose(-1, -2) / math.sqrt(128)
     ref = torch.softmax(logits.masked_fill(~(allowed & causal), float("-inf")), -1) @ vf
     assert_attn_close(out, ref, what=f"B={B} Hq={Hq} S={S}")
+
+
+def test_tile_pipeline_probe_runs_and_reports_clocks(dev):
+    """The measurement entry point: a short run on zero and on random tiles returns finite sums and both clock counters."""
+    from pbs_attn_amd import _lib
+    lib = _lib.load()
+    sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
+    st = torch.cuda.current_stream().cuda_stream
+    for ring in (torch.zeros(4 * 32768, dtype=torch.bfloat16, device=dev),
+                 torch.randn(4 * 32768, generator=torch.Generator().manual_seed(3)).to(torch.bfloat16).to(dev)):
+        for copies in (0, 1):
+            clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+            _lib.check(lib.pbs_attn_tile_probe(ring.data_ptr(), 4, 50, copies, sink.data_ptr(), clocks.data_ptr(), st), "probe")
+            torch.cuda.synchronize()
+            c = clocks.tolist()
+            assert torch.isfinite(sink).all() and c[0] > 50 * 4096 and c[1] > 0   # at least the matrix pipe's cycles per tile
+    assert lib.pbs_attn_tile_probe(None, 4, 50, 0, sink.data_ptr(), clocks.data_ptr(), st) < 0
