@@ -53,21 +53,59 @@ __device__ __forceinline__ f32x2 logit2(float acc0, float acc1, float inv_sqrt_d
 }
 constexpr float LOG2E = 1.4426950408889634f;
 
-// One wave per query head of the KV group; the four waves of a workgroup walk
-// the same key chunk so K comes out of the CU's L1 after the first wave.
+// ---- key rows through LDS: the waves of a workgroup (one per query head of the KV group) walk the same keys,
+// so a stage of 64 key rows is copied once per workgroup with asynchronous global -> LDS copies (no registers),
+// double-buffered, and every wave reads its MFMA fragments from there.  Rows are 16 chunks of 16 bytes with the
+// chunk index XORed with (row & 15): fragment reads (row = lane % 32, one chunk) are bank-conflict free.  The copy
+// instruction writes lane l at M0 + 16 l, so the swizzle is applied on the global side: lane l of copy i fetches
+// chunk (l & 15) ^ (row & 15) of row 4 i + (l >> 4).
+constexpr int STAGE_KEYS = 64;
+constexpr uint32_t STAGE_BYTES = STAGE_KEYS * D * 2;      // 16 KB
+constexpr uint32_t LDS_STATS = 2 * STAGE_BYTES;           // per wave: NQ floats (row max + log2 row sum)
+constexpr uint32_t LDS_SCORE_TOTAL = LDS_STATS + 4 * NQ * 4;
+
+typedef __attribute__((address_space(3))) uint8_t lds_u8;
+
+__device__ __forceinline__ bf16x8 lds_frag(uint32_t byte_addr) {
+  return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const lds_u8*)(uintptr_t)byte_addr);
+}
+
+// copies of rows [0, STAGE_KEYS) starting at `rows` (row stride k_ss elements) into the stage buffer at LDS byte
+// offset `lds_byte`; wave w of nwaves issues copies w, w + nwaves, ...
+__device__ __forceinline__ void stage_keys_async(const uint16_t* rows, int64_t k_ss, uint32_t lds_byte, int wave, int nwaves, int lane) {
+  const uint64_t src0 = (uint64_t)(uintptr_t)rows;
+  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
+  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
+  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
+  const uint32_t row_bytes = (uint32_t)k_ss * 2u;   // < 2^29 (checked on the host)
+  for (int i = wave; i < STAGE_KEYS / 4; i += nwaves) {
+    const uint32_t r = (uint32_t)(lane >> 4);
+    const uint32_t c = (uint32_t)(lane & 15) ^ ((4u * (uint32_t)(i & 3) + r) & 15u);
+    const uint32_t voff = r * row_bytes + c * 16u;
+    const uint64_t base = srcu + (uint64_t)(4 * i) * row_bytes;
+    register uint32_t m0v asm("m0") = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + (uint32_t)i * 1024u));
+    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base) : "memory");
+  }
+}
+
+// One wave per query head of the KV group; the waves of a workgroup share the staged key rows.
 template <bool FINAL>
-__global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+__global__ __launch_bounds__(256, 2) void score_kernel(ScoreArgs a) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // starts at LDS offset 0: this kernel has no static LDS
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   const int j = lane & 31, half = lane >> 5;
   const int G = a.Hq / a.Hkv;
   const int b = blockIdx.y / a.Hkv, kvh = blockIdx.y % a.Hkv;
   const int chunk = blockIdx.x;
   const int key_lo = chunk * a.chunk_keys;
-  const int key_hi = min(key_lo + a.chunk_keys, a.Sc);
-  const int nwaves = blockDim.x >> 6;
+  const int key_hi = min(key_lo + a.chunk_keys, a.Sc);   // chunk_keys and Sc are multiples of STAGE_KEYS
+  const int nwaves = (int)blockDim.x >> 6;
   const uint16_t* kbase = a.k + b * a.k_sb + kvh * a.k_sh;
-
-  __shared__ float s_stats[4][NQ];   // per query row: max + log2(sum), so that p = exp2(logit - stat)
+  float* s_stats = reinterpret_cast<float*>(smem + LDS_STATS) + wave * NQ;   // p = exp2(logit - stat)
+  // LDS byte offset of fragment 0 of key row j inside a stage buffer; fragment t lies at frag0 ^ (t << 5),
+  // rows 32 .. 63 of the stage 8 KB further on
+  const uint32_t frag0 = (uint32_t)(j * 256 + ((half ^ (j & 15)) * 16));
+  const int n_stages = (key_hi - key_lo) / STAGE_KEYS;
 
   for (int g0 = 0; g0 < G; g0 += nwaves) {
     const int g = g0 + wave;
@@ -76,6 +114,9 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
     const int bh = b * a.Hq + h;
     const uint16_t* qbase = a.q + b * a.q_sb + h * a.q_sh + (int64_t)(a.S - NQ) * a.q_ss;
 
+    __syncthreads();   // every wave is done with the stage buffers (and the statistics) of the previous group of heads
+    stage_keys_async(kbase + (int64_t)key_lo * a.k_ss, a.k_ss, 0u, wave, nwaves, lane);
+
     // the head's 128 scoring queries, resident for the whole chunk
     bf16x8 qf[4][8];
 #pragma unroll
@@ -83,12 +124,8 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
 #pragma unroll
       for (int t = 0; t < 8; ++t) qf[qt][t] = load_frag(qbase + (int64_t)(32 * qt + j) * a.q_ss, t, half);
 
-    if (FINAL) {
-      __syncthreads();
-      if (active)
-        for (int i = lane; i < NQ; i += 64) s_stats[wave][i] = a.stats[(int64_t)bh * NQ + i];
-      __syncthreads();
-    }
+    if (FINAL && active)
+      for (int i = lane; i < NQ; i += 64) s_stats[i] = a.stats[(int64_t)bh * NQ + i];
 
     float m_run[4], l_run[4];
 #pragma unroll
@@ -97,24 +134,19 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
       l_run[qt] = 0.f;
     }
 
-    if (active) {
-      // the next step's key rows are in flight while this step computes
-      bf16x8 kf_next[8];
-      {
-        const uint16_t* krow = kbase + (int64_t)(key_lo + j) * a.k_ss;
+    for (int st = 0; st < n_stages; ++st) {
+      const uint32_t buf = (uint32_t)(st & 1) * STAGE_BYTES;
+      __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this wave's copies of stage st have landed
+      __syncthreads();                      // every wave's have; everyone is done with the other buffer
+      if (st + 1 < n_stages)
+        stage_keys_async(kbase + (int64_t)(key_lo + (st + 1) * STAGE_KEYS) * a.k_ss, a.k_ss, buf ^ STAGE_BYTES, wave, nwaves, lane);
+      if (!active) continue;
 #pragma unroll
-        for (int t = 0; t < 8; ++t) kf_next[t] = load_frag(krow, t, half);
-      }
-      for (int key0 = key_lo; key0 < key_hi; key0 += KEYS_PER_WAVE_STEP) {
-        const int key = key0 + j;  // always < Sc: Sc is a multiple of 128
+      for (int sub = 0; sub < STAGE_KEYS / KEYS_PER_WAVE_STEP; ++sub) {
+        const int key = key_lo + st * STAGE_KEYS + sub * KEYS_PER_WAVE_STEP + j;   // always < Sc
         bf16x8 kf[8];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) kf[t] = kf_next[t];
-        if (key0 + KEYS_PER_WAVE_STEP < key_hi) {
-          const uint16_t* krow = kbase + (int64_t)(key + KEYS_PER_WAVE_STEP) * a.k_ss;
-#pragma unroll
-          for (int t = 0; t < 8; ++t) kf_next[t] = load_frag(krow, t, half);
-        }
+        for (int t = 0; t < 8; ++t) kf[t] = lds_frag(buf + (uint32_t)sub * 8192u + (frag0 ^ (uint32_t)(t << 5)));
 
         if (!FINAL) {
           // S^T tile: rows = keys, column = query j of sub-tile qt
@@ -148,30 +180,30 @@ __global__ __launch_bounds__(256) void score_kernel(ScoreArgs a) {
             for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qf[qt][t], kf[t], acc, 0, 0, 0);
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4) {
-              const float4 st = *reinterpret_cast<const float4*>(&s_stats[wave][32 * qt + 8 * r4 + 4 * half]);
+              const float4 st4 = *reinterpret_cast<const float4*>(&s_stats[32 * qt + 8 * r4 + 4 * half]);
               const f32x2 la = logit2(acc[4 * r4 + 0], acc[4 * r4 + 1], a.inv_sqrt_d);
               const f32x2 lb = logit2(acc[4 * r4 + 2], acc[4 * r4 + 3], a.inv_sqrt_d);
-              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.x, LOG2E, -st.x));
-              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.y, LOG2E, -st.y));
-              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.x, LOG2E, -st.z));
-              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.y, LOG2E, -st.w));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.x, LOG2E, -st4.x));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(la.y, LOG2E, -st4.y));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.x, LOG2E, -st4.z));
+              accp += __builtin_amdgcn_exp2f(__builtin_fmaf(lb.y, LOG2E, -st4.w));
             }
           }
           accp += xhalf_f32(accp);
           if (half == 0) a.scores[(int64_t)bh * a.Sc + key] = accp * (1.0f / NQ);
         }
       }
-      if (!FINAL) {
+    }
+    if (!FINAL && active) {
 #pragma unroll
-        for (int qt = 0; qt < 4; ++qt) {
-          const float m_o = xhalf_f32(m_run[qt]), l_o = xhalf_f32(l_run[qt]);
-          const float m_new = fmaxf(m_run[qt], m_o);
-          const float l_new = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + l_o * __builtin_amdgcn_exp2f(m_o - m_new);
-          if (half == 0) {
-            float* p = a.part + (((int64_t)bh * a.nchunk + chunk) * NQ + 32 * qt + j) * 2;
-            p[0] = m_new;
-            p[1] = l_new;
-          }
+      for (int qt = 0; qt < 4; ++qt) {
+        const float m_o = xhalf_f32(m_run[qt]), l_o = xhalf_f32(l_run[qt]);
+        const float m_new = fmaxf(m_run[qt], m_o);
+        const float l_new = l_run[qt] * __builtin_amdgcn_exp2f(m_run[qt] - m_new) + l_o * __builtin_amdgcn_exp2f(m_o - m_new);
+        if (half == 0) {
+          float* p = a.part + (((int64_t)bh * a.nchunk + chunk) * NQ + 32 * qt + j) * 2;
+          p[0] = m_new;
+          p[1] = l_new;
         }
       }
     }
@@ -229,6 +261,7 @@ int score_keys_launch(const char* who, const void* q, const void* k, float* scor
   PBS_REQUIRE(q_ss % 8 == 0 && k_ss % 8 == 0 && q_sh % 8 == 0 && k_sh % 8 == 0 && q_sb % 8 == 0 && k_sb % 8 == 0,
               "%s: strides must keep rows 16-byte aligned", who);
   PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0, "%s: pointers must be 16-byte aligned", who);
+  PBS_REQUIRE(k_ss >= D && k_ss < (1 << 28), "%s: key row stride %lld outside [128, 2^28)", who, (long long)k_ss);
   PBS_REQUIRE((int64_t)B * Hkv <= 65535, "%s: too many KV heads (%lld)", who, (long long)B * Hkv);
   const int Sc = (S / segment_size) * segment_size;
   if (Sc == 0) return 0;
@@ -250,9 +283,9 @@ int score_keys_launch(const char* who, const void* q, const void* k, float* scor
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(a.nchunk, B * Hkv);
   const dim3 block(Hq / Hkv > 1 ? 256 : 64);
-  hipLaunchKernelGGL(score_kernel<false>, grid, block, 0, st, a);
+  hipLaunchKernelGGL(score_kernel<false>, grid, block, LDS_SCORE_TOTAL, st, a);
   hipLaunchKernelGGL(score_reduce_kernel, dim3(B * Hq), dim3(NQ), 0, st, a);
-  hipLaunchKernelGGL(score_kernel<true>, grid, block, 0, st, a);
+  hipLaunchKernelGGL(score_kernel<true>, grid, block, LDS_SCORE_TOTAL, st, a);
   return pbs_check_launch(who);
 }
 
