@@ -29,7 +29,8 @@ const char* pbs_last_error(void);
 
 /* Key scoring: scores[b,h,k] = mean over the last 128 queries of
  * softmax_k(bf16(bf16(q.k) / sqrt(D))) over the keys of the complete segments.
- * scores: (B, Hq, Sc) float32, Sc = (S / segment_size) * segment_size.
+ * scores: (B, Hq, Sc) float32, Sc = (S / segment_size) * segment_size.  Strides in elements, rows 16-byte
+ * aligned, key row stride in [128, 2^28).
  * Replaces pbs_attn/src/permute_states.py:44-50. */
 size_t pbs_score_keys_workspace_bytes(int B, int Hq, int Hkv, int S, int segment_size);
 int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, int Hkv, int S, int head_dim,

@@ -1,7 +1,7 @@
 // Key scoring: mean over the last 128 queries of softmax(Q_last K^T / sqrt(D))
 // over all keys of the complete segments (no causal mask).
 //
-// Three launches, K is read twice and never re-materialised:
+// Three launches, K is read twice (each time once per workgroup, through LDS) and never re-materialised:
 //   (all exponentials are base 2 on logits pre-multiplied by log2(e))
 //   1. score_partial : per (head, key chunk) online (max, sum-exp) of every query row
 //   2. score_reduce  : fold the chunk partials into row max + log2(row sum)
