@@ -75,6 +75,10 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert rc < 0 and b"head_dim" in lib.pbs_last_error()
     with pytest.raises(_lib.PbsHipError):
         _lib.check(rc, "pbs_pool_q")
+    # a key row stride the scoring kernel's 32-bit copy offsets cannot hold (pointers are only checked, never read)
+    fake = 4096
+    rc = lib.pbs_score_keys(fake, fake, fake, 1, 4, 2, 1024, 128, 128, 256, 0, 0, 128, 0, 0, 1 << 28, fake, 1 << 30, None)
+    assert rc < 0 and b"key row stride" in lib.pbs_last_error()
 
 
 def test_reference_import_paths():
