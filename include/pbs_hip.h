@@ -151,6 +151,19 @@ int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, 
                         int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
                         float softmax_scale, void* workspace, void* stream);
 
+/* pbs_sparse_attn_fwd for one-block segments (segment_size = block_size: the un-permuted MeanPooling mode) with an
+ * OPTIONAL diagonal block: query block qb of head row r attends to its own block (with the causal triangle) only
+ * where own_block_needed[r * nb + qb] != 0 ((B*Hq, nb) bytes), and to the blocks of csr_cols as before.  Every
+ * query block must be left with at least one block.  Workspace: pbs_sparse_attn_workspace_bytes(B, Hq, S,
+ * block_size).  Replaces the attention call of pbs_attn/baselines/MeanPooling.py:80-96 when
+ * force_select_current_block (:54-58) is off. */
+int pbs_sparse_attn_fwd_optional_diagonal(const void* q, const void* perm_k, const void* perm_vt, const void* k,
+                                          const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt,
+                                          const uint8_t* own_block_needed, void* out, int B, int Hq, int Hkv, int S,
+                                          int head_dim, int block_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                          int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh,
+                                          int64_t o_ss, float softmax_scale, void* workspace, void* stream);
+
 /* out[b,h,q_idx[b,h,i],:] = o_perm[b,h,i,:] (o_perm contiguous).  q_idx null with
  * o_perm == out is the identity fast path (no launch): the reference does not
  * permute queries (pbs_attn/src/pbs.py:191-193), so this is what it takes. */

@@ -27,6 +27,7 @@ SIGNATURES = {
     "pbs_select_blocks": (c_int, [_P, _P, _F, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "pbs_sparse_attn_workspace_bytes": (c_size_t, [_I] * 4),
     "pbs_sparse_attn_fwd": (c_int, [_P] * 8 + [_I] * 7 + [_L] * 9 + [_F, _P, _P]),
+    "pbs_sparse_attn_fwd_optional_diagonal": (c_int, [_P] * 9 + [_I] * 6 + [_L] * 9 + [_F, _P, _P]),
     "pbs_unpermute": (c_int, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
     "pbs_rope_qk": (c_int, [_P] * 6 + [_I] * 5 + [_L] * 8 + [_P]),
     "pbs_mfma_probe": (c_int, [_P, _I, _P, _P, _P]),

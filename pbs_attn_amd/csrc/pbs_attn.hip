@@ -251,7 +251,7 @@ __device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8],
 // the work counters of the attention kernel that follows on the stream.
 __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __restrict__ cols, const int32_t* __restrict__ cnt,
                                                                uint16_t* __restrict__ plist, int* __restrict__ queue, int nb,
-                                                               int bps, int cap) {
+                                                               int bps, int cap, const uint8_t* __restrict__ own_needed) {
   __shared__ uint8_t flags0[4096], flags1[4096];
   __shared__ int wsum[8];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -311,6 +311,16 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
   const int qb0 = 2 * pair, qb1 = second ? qb0 + 1 : qb0;
   const int sf0 = (qb0 / bps) * bps, sf1 = (qb1 / bps) * bps;
   const int n_own = qb1 - sf0 + 1;
+  if (own_needed) {
+    // one-block segments with an optional diagonal: a query block's own block is listed only where its flag is set
+    if (tid == 0) {
+      int n = total;
+      if (own_needed[(int64_t)bh * nb + qb0]) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG | (1u << 14));
+      if (second && own_needed[(int64_t)bh * nb + qb1]) out[1 + n++] = (uint16_t)(qb1 | ENT_ORIG | (2u << 14));
+      out[0] = (uint16_t)n;
+    }
+    return;
+  }
   if (tid < n_own) {
     const int kb = sf0 + tid;
     const int f = (kb <= qb0 ? 1 : 0) | ((second && kb >= sf1) ? 2 : 0);
@@ -789,11 +799,39 @@ extern "C" size_t pbs_sparse_attn_workspace_bytes(int B, int Hq, int S, int segm
   return 256 + (size_t)B * Hq * npair * cap * 2;
 }
 
+static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+                              const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
+                              int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                              float softmax_scale, const uint8_t* own_block_needed, void* workspace, void* stream);
+
 extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k,
                                    const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B,
                                    int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size, int64_t q_sb,
                                    int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb,
                                    int64_t o_sh, int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
+  return sparse_attn_launch(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size,
+                            segment_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, nullptr,
+                            workspace, stream);
+}
+
+extern "C" int pbs_sparse_attn_fwd_optional_diagonal(const void* q, const void* perm_k, const void* perm_vt, const void* k,
+                                                     const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt,
+                                                     const uint8_t* own_block_needed, void* out, int B, int Hq, int Hkv, int S,
+                                                     int head_dim, int block_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                                     int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh,
+                                                     int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
+  PBS_REQUIRE(own_block_needed, "pbs_sparse_attn_fwd_optional_diagonal: null own_block_needed");
+  return sparse_attn_launch(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size,
+                            block_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, own_block_needed,
+                            workspace, stream);
+}
+
+static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+                              const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
+                              int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
+                              float softmax_scale, const uint8_t* own_block_needed, void* workspace, void* stream) {
   PBS_REQUIRE(q && perm_k && perm_vt && k && orig_vt && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
   PBS_REQUIRE(workspace && ((uintptr_t)workspace % 256) == 0, "pbs_sparse_attn_fwd: workspace must be a 256-byte aligned device buffer of pbs_sparse_attn_workspace_bytes()");
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_sparse_attn_fwd: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
@@ -862,7 +900,7 @@ extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void
     return (int)attr;
   }
   hipLaunchKernelGGL(merge_pair_lists_kernel, dim3((unsigned)(a.BH * npair)), dim3(512), 0, (hipStream_t)stream, csr_cols, csr_cnt,
-                     (uint16_t*)((char*)workspace + 256), a.queue, a.nb, a.bps, a.cap);
+                     (uint16_t*)((char*)workspace + 256), a.queue, a.nb, a.bps, a.cap, own_block_needed);
   hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(512), LDS_TOTAL, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_sparse_attn_fwd");
 }

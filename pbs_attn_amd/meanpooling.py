@@ -10,8 +10,8 @@ here the identity key order goes through the same gather / estimate / select / a
 every selected earlier block is read unmasked).
 
 Differences a caller can see: any batch size and K/V at the KV-head count are accepted (the
-reference asserts batch 1 and expanded heads); ``force_select_current_block=False`` is not built
-(the attention kernel always attends to the diagonal block)."""
+reference asserts batch 1 and expanded heads).  With ``force_select_current_block=False`` a query block
+attends to its diagonal block only where the threshold selected it (MeanPooling.py:54-58)."""
 from __future__ import annotations
 
 import torch
@@ -36,9 +36,6 @@ def MeanPooling_prefill(
     assert num_q_heads % num_kv_heads == 0
     assert q_len == kv_len, "Only support prefilling for now, q_len: {}, kv_len: {}".format(q_len, kv_len)
     assert causal
-    if not force_select_current_block:
-        raise NotImplementedError("MeanPooling_prefill: force_select_current_block=False is not built: the HIP "
-                                  "attention kernel always attends to a query block's diagonal block")
     s_pad = (q_len + block_size - 1) // block_size * block_size
     idx = torch.arange(s_pad, dtype=torch.int32, device=query_states.device).view(1, 1, -1)
     idx = idx.expand(batch_size, num_q_heads, -1).contiguous()
@@ -50,9 +47,15 @@ def MeanPooling_prefill(
     thr = threshold if isinstance(threshold, torch.Tensor) else float(threshold)
     # one block per segment: the visit list holds the selected blocks before the diagonal, the diagonal
     # block (MeanPooling.py:54-58) is the attention kernel's own-segment tile
-    sel, fin, cols, cnt = ops.select_blocks(scores, thr, idx, q_len, block_size, block_size,
-                                            force_select_first_block, want_masks=return_masks, candidate_rule=2)
-    out = ops.sparse_attn_fwd(query_states, perm_k, perm_vt, key_states, orig_vt, cols, cnt, block_size)
+    sel, fin, cols, cnt = ops.select_blocks(scores, thr, idx, q_len, block_size, block_size, force_select_first_block,
+                                            want_masks=return_masks or not force_select_current_block, candidate_rule=2)
+    own = None
+    if not force_select_current_block:
+        # the diagonal block only where the threshold chose it (or it is block 0 and that one is forced): the plain
+        # selection mask says where
+        fin = sel   # the selection with the forced first column, without the forced diagonal
+        own = fin.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
+    out = ops.sparse_attn_fwd(query_states, perm_k, perm_vt, key_states, orig_vt, cols, cnt, block_size, own_block_needed=own)
     if return_masks:
         return out, dict(block_attn_scores=scores, block_mask=fin, csr_cnt=cnt)
     return out

@@ -224,10 +224,12 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     return sel, fin, cols, cnt
 
 
-def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
+def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None,
+                    own_block_needed=None):
     """Attention of every query block over the permuted tiles listed in the CSR (earlier segments) and
     over the causal part of its own segment, read from the original ``k`` (B, Hkv or Hq, S, D) and
-    ``orig_vt``."""
+    ``orig_vt``.  ``own_block_needed`` ((B, Hq, nb) uint8, one-block segments only) makes the diagonal block
+    optional per query block."""
     _check_bf16_cuda(q, perm_k, perm_vt, k, orig_vt)
     lib = _lib.load()
     q, k = _rows16(q), _rows16(k)
@@ -244,6 +246,15 @@ def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_s
     assert csr_cols.is_contiguous() and csr_cnt.is_contiguous()
     assert csr_cols.shape == (B, Hq, nb, nb) and csr_cnt.shape == (B, Hq, nb)
     ws = torch.empty(max(lib.pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size), 256), dtype=torch.uint8, device=q.device)
+    if own_block_needed is not None:
+        if segment_size != BLOCK:
+            raise ValueError("own_block_needed: only for one-block segments (segment_size == block_size)")
+        assert own_block_needed.shape == (B, Hq, nb) and own_block_needed.dtype == torch.uint8 and own_block_needed.is_contiguous()
+        _lib.check(lib.pbs_sparse_attn_fwd_optional_diagonal(
+            _ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols), _ptr(csr_cnt), _ptr(own_block_needed),
+            _ptr(out), B, Hq, Hkv, S, D, BLOCK, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+            out.stride(0), out.stride(1), out.stride(2), softmax_scale, _ptr(ws), _stream()), "pbs_sparse_attn_fwd_optional_diagonal")
+        return out
     _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols),
                                        _ptr(csr_cnt), _ptr(out), B, Hq, Hkv, S, D, BLOCK, segment_size,
                                        q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),

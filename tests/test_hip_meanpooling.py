@@ -56,8 +56,45 @@ def test_meanpooling_through_the_factory_and_patch(dev):
     fn = get_meanpooling_prefill(threshold=0.9)
     out = fn(q.to(dev), k.to(dev), v.to(dev))
     assert out.shape == q.shape and torch.isfinite(out.float()).all()
-    with pytest.raises(NotImplementedError):
-        get_meanpooling_prefill(force_select_current_block=False)(q.to(dev), k.to(dev), v.to(dev))
+    out = get_meanpooling_prefill(force_select_current_block=False)(q.to(dev), k.to(dev), v.to(dev))
+    assert out.shape == q.shape and torch.isfinite(out.float()).all()
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,thr,ff", [(1, 4, 2, 2048, 0.3, True), (2, 2, 2, 1000, 0.5, True), (1, 7, 1, 1536, 0.2, False),
+                                               (1, 2, 2, 1280, 0.9, True)])
+def test_meanpooling_with_an_optional_diagonal_block(dev, B, Hq, Hkv, S, thr, ff):
+    """force_select_current_block=False (MeanPooling.py:54-58 skipped): a query block attends to its diagonal block
+    only where the threshold selected it.  Masks bit-exact on the oracle's block probabilities, output against dense
+    attention on that mask; low thresholds so that many diagonals are in fact dropped."""
+    q, k, v = small_case(B, Hq, Hkv, S, seed=S + Hq + 1)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref_out, mid = O.meanpooling_prefill(q, ke, ve, 128, 1024, thr, True, ff, False, return_intermediates=True)
+    nb = (S + 127) // 128
+    eye = torch.eye(nb, dtype=torch.bool)
+    dropped = (~mid["block_mask"] & eye).sum().item()
+    if thr < 0.9:
+        assert dropped > 0, "the case is meant to drop diagonal blocks"
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    idx = torch.arange(nb * 128, dtype=torch.int32, device=dev).view(1, 1, -1).expand(B, Hq, -1).contiguous()
+    sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, ff, candidate_rule=2)
+    assert torch.equal(sel.cpu(), mid["block_mask"])
+    own = sel.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=own).cpu()
+    dense = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128)
+    assert_attn_close(out, dense, what="optional diagonal: HIP vs dense fp32 on the oracle's mask")
+    assert_attn_close(ref_out, dense, max_abs=2.5e-2, what="oracle naive vs dense fp32")
+    # with every flag set the entry point is the plain one
+    ones = torch.ones_like(own)
+    a = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=ones)
+    b = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128)
+    assert torch.equal(a, b)
+    # the whole mode from raw Q, K, V
+    out2, got = MeanPooling_prefill(qd, kd, vd, 128, 1024, thr, True, ff, False, return_masks=True)
+    own_mask = got["block_mask"].cpu()
+    assert (own_mask == mid["block_mask"]).float().mean().item() >= 0.99
+    dense2 = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], own_mask, 128)
+    assert_attn_close(out2.cpu(), dense2, what="MeanPooling_prefill (optional diagonal) vs dense fp32 on its own mask")
 
 
 def test_stage_adapters_with_the_reference_signatures(dev):
