@@ -75,6 +75,7 @@ struct AttnArgs {
   int BH, Hq, Hkv, S, nb, bps;
   uint32_t k_ss;   // key row stride in elements (< 2^22)
   int xcd_start[9];   // work items (head-major, long rows first) of XCD x: [xcd_start[x], xcd_start[x + 1])
+  int interleave;     // 0, or 1 + log2(whole heads per XCD range) of a small launch whose tickets go pair-major (see ticket_item)
   int64_t q_sb, q_sh, q_ss, k_sb, k_sh, o_sb, o_sh, o_ss;
   float scale_log2;
 };
@@ -329,6 +330,21 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
   if (tid == 0) out[0] = (uint16_t)(total + n_own);
 }
 
+// Ticket t of the counter of a range of `count` items starting at `begin` -> work item.  Items are numbered head by
+// head, long rows first, and normally handed out in that order (an XCD walks one head at a time: its workgroups
+// share that head's K / V stream in L2).  A launch with only a few items per workgroup cannot balance that way: a
+// workgroup that starts with a short item of one head is handed a long item of the next and finishes last.  There
+// (`il` = 1 + log2 of the whole heads per range, a power of two) the same row pair of every head of the range goes
+// out before the next shorter pair: longest items first across the range.
+// Takes and returns begin + ticket (wave-uniform values: scalar arithmetic only); a ticket past the range is left alone.
+__device__ __forceinline__ int ticket_item(int begin, int end, int item, int il, int npair) {
+  if (il > 0 && item < end) {
+    const int t = item - begin;
+    item = begin + (t & ((1 << (il - 1)) - 1)) * npair + (t >> (il - 1));
+  }
+  return item;
+}
+
 // asynchronous copy of one list row (`chunks` 16-byte pieces) into LDS at byte offset `lds_byte`
 __device__ __forceinline__ void stage_list_async(const uint16_t* src, int chunks, uint32_t lds_byte, int wave, int tid) {
   const uint64_t src0 = (uint64_t)(uintptr_t)src;
@@ -371,7 +387,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     misc[1] = 0;
   }
   __syncthreads();
-  int cur = __builtin_amdgcn_readfirstlane(misc[2]);
+  int cur = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[2]), a0->interleave, npair);
   if (cur >= q_end) return;
   int nxt = q_end;   // the next item is claimed late in the current one: an item claimed early waits for this
                      // workgroup while others may be idle
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       if (wave == 0 && lane_id_here() == 0) misc[4] = q_begin + claim;
     };
     auto adopt_next = [&]() {          // ... and after the barrier
-      nxt = __builtin_amdgcn_readfirstlane(misc[4]);
+      nxt = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[4]), PBS_ARGS()->interleave, npair);
       has_nxt = nxt < q_end;
       if (has_nxt) {
         ArgsPtr an = PBS_ARGS();
@@ -696,7 +712,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         __syncthreads();   // everyone has read the previous ticket
         if (wave == 0 && lane_id_here() == 0) misc[4] = q_begin + atomicAdd(as->queue + vic, 1);
         __syncthreads();
-        nxt = __builtin_amdgcn_readfirstlane(misc[4]);
+        nxt = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[4]), as->interleave, npair);
         if (nxt < q_end) {
           has_nxt = true;
           break;
@@ -874,6 +890,13 @@ static int sparse_attn_launch(const void* q, const void* perm_k, const void* per
     if (x == 8) start = (int64_t)a.BH * npair;
     a.xcd_start[x] = (int)start;
     if (x > 0) max_items = std::max(max_items, a.xcd_start[x] - a.xcd_start[x - 1]);
+  }
+  // few items per workgroup and ranges of whole heads: hand the tickets out pair-major (see ticket_item)
+  a.interleave = 0;
+  const int nh = a.BH / 8;
+  if (a.BH % 8 == 0 && (nh & (nh - 1)) == 0 && (int64_t)a.BH * npair <= (int64_t)8 * 256) {
+    for (a.interleave = 1; (1 << (a.interleave - 1)) < nh; ++a.interleave) {}
+    for (int x = 0; x <= 8; ++x) a.xcd_start[x] = (int)(x * (int64_t)nh * npair);
   }
   a.cap = list_cap(a.nb, a.bps);
   PBS_REQUIRE((uint32_t)a.cap * 2 <= LIST_BYTES, "pbs_sparse_attn_fwd: visit list too long");
