@@ -891,10 +891,11 @@ static int sparse_attn_launch(const void* q, const void* perm_k, const void* per
     a.xcd_start[x] = (int)start;
     if (x > 0) max_items = std::max(max_items, a.xcd_start[x] - a.xcd_start[x - 1]);
   }
-  // few items per workgroup and ranges of whole heads: hand the tickets out pair-major (see ticket_item)
+  // at most two items per workgroup and ranges of whole heads: hand the tickets out pair-major (see ticket_item;
+  // with four and more items per workgroup the head-by-head order balances well enough and is 1-3 % faster)
   a.interleave = 0;
   const int nh = a.BH / 8;
-  if (a.BH % 8 == 0 && (nh & (nh - 1)) == 0 && (int64_t)a.BH * npair <= (int64_t)8 * 256) {
+  if (a.BH % 8 == 0 && (nh & (nh - 1)) == 0 && (int64_t)a.BH * npair <= (int64_t)2 * 256) {
     for (a.interleave = 1; (1 << (a.interleave - 1)) < nh; ++a.interleave) {}
     for (int x = 0; x <= 8; ++x) a.xcd_start[x] = (int)(x * (int64_t)nh * npair);
   }

@@ -39,7 +39,7 @@ def test_short_sequences_every_block_selected(dev, S, seg):
     (4, 8, 2, 2048, 256, 0.3),       # 256 short items
     (1, 1, 1, 16384 + 128, 256, 0.9),  # one head, odd block count: the last item is a single query block
     (1, 32, 8, 4096, 256, 0.9),      # few items per workgroup, 4 whole heads per range: tickets handed out pair-major
-    (2, 8, 8, 2048 + 300, 512, 0.7),   # same with 2 heads per range, ragged length, odd block count
+    (2, 8, 8, 2048 + 300, 512, 0.7),   # same with 2 heads per range, ragged length, odd block count (160 items)
     (1, 8, 2, 1024, 256, 0.9),       # one head per range: pair-major is head-major
 ])
 def test_work_distribution_shapes_against_dense_attention_on_the_mask(dev, B, Hq, Hkv, S, seg, thr):
