@@ -675,3 +675,35 @@ def test_both_poolings_in_one_launch_are_the_same_bits(dev, Hq, Hkv, S, seg, qmo
     assert torch.equal(pq, ops.pool_q(qd, qmode))
     assert torch.equal(pk, ops.pool_k_permuted(kd, idx, Hq, kmode)[0])
     assert int(needed.sum()) == 0
+
+
+def test_single_call_operator_under_hip_graph_capture(dev):
+    """The whole-path call allocates nothing itself, synchronises nothing and records no memset node: captured into a
+    HIP graph it replays to the eager bits, replay after replay, with eager work and synchronisations in between."""
+    q, k, v = small_case(1, 4, 2, 2048 + 77, kind="strong_heavy", seed=83)
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+
+    def step(x):
+        return ops.prefill_attn_fwd(x, kd, vd, 128, 512, 0.8)
+
+    ref = step(qd)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(qd)
+    torch.cuda.current_stream().wait_stream(side)
+    static_q = qd.clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = step(static_q)
+    torch.cuda.synchronize()
+    q2 = (qd.float() * 0.5).to(torch.bfloat16)
+    ref2 = step(q2)
+    for rep in range(4):
+        static_q.copy_(q2 if rep % 2 else qd)       # new inputs through the captured buffer
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, ref2 if rep % 2 else ref), rep
+        assert torch.equal(step(qd), ref)           # eager work between the replays
+        torch.cuda.synchronize()
