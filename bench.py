@@ -80,13 +80,33 @@ class StageTimer:
         return {k: sum(v) / len(v) for k, v in tot.items()}
 
 
+_probe_lib = None
+
+
+def load_probe_library():
+    """libpbs_probe.so: the measurement kernels (an MFMA-only loop, the attention kernel's tile pipeline alone).
+    Bench-only: built next to the operator's library, not part of its ABI."""
+    global _probe_lib
+    if _probe_lib is None:
+        import ctypes
+        from ctypes import c_double, c_int, c_void_p
+        from pbs_attn_amd import _lib
+        _lib.load()   # the probe library takes its error helpers from the operator's library
+        lib = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libpbs_probe.so"))
+        lib.pbs_mfma_probe.restype, lib.pbs_mfma_probe.argtypes = c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]
+        lib.pbs_mfma_probe_flop.restype, lib.pbs_mfma_probe_flop.argtypes = c_double, [c_int]
+        lib.pbs_attn_tile_probe.restype = c_int
+        lib.pbs_attn_tile_probe.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
+        _probe_lib = lib
+    return _probe_lib
+
+
 def mfma_ceiling(torch, iters=200000):
     """What a loop of nothing but bf16 MFMAs sustains on this GPU right now, on all-zero operands and on
     normally distributed ones (the rate depends on the values: the chip lowers its clock to stay inside its
     power limit).  The second figure is the practical ceiling for a kernel fed with data like attention's."""
-    import ctypes
     from pbs_attn_amd import _lib
-    lib = _lib.load()
+    lib = load_probe_library()
     dev = torch.device("cuda")
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     gen = torch.Generator(device="cpu").manual_seed(7)
@@ -118,7 +138,7 @@ def tile_pipeline(torch, iters=6000):
     the clock falls with the power limit; what the attention kernel reaches of this rate is the cost of
     everything around the pipeline."""
     from pbs_attn_amd import _lib
-    lib = _lib.load()
+    lib = load_probe_library()
     dev = torch.device("cuda")
     n_src = 256                                     # 16 MB ring of tile pairs
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)

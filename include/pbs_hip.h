@@ -153,8 +153,9 @@ int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, 
 
 /* pbs_sparse_attn_fwd for one-block segments (segment_size = block_size: the un-permuted MeanPooling mode) with an
  * OPTIONAL diagonal block: query block qb of head row r attends to its own block (with the causal triangle) only
- * where own_block_needed[r * nb + qb] != 0 ((B*Hq, nb) bytes), and to the blocks of csr_cols as before.  Every
- * query block must be left with at least one block.  Workspace: pbs_sparse_attn_workspace_bytes(B, Hq, S,
+ * where own_block_needed[r * nb + qb] != 0 ((B*Hq, nb) bytes), and to the blocks of csr_cols as before.  A query
+ * block left without any block gets zeros, like a row without selected blocks in
+ * pbs_attn/src/kernels/permuted_block_sparse_attention.py:340-343.  Workspace: pbs_sparse_attn_workspace_bytes(B, Hq, S,
  * block_size).  Replaces the attention call of pbs_attn/baselines/MeanPooling.py:80-96 when
  * force_select_current_block (:54-58) is off. */
 int pbs_sparse_attn_fwd_optional_diagonal(const void* q, const void* perm_k, const void* perm_vt, const void* k,
@@ -196,24 +197,6 @@ int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v, void* out,
 int pbs_rope_qk(const void* q, const void* k, const void* cos, const void* sin, void* q_out, void* k_out, int B, int Hq,
                 int Hkv, int S, int head_dim, int64_t q_sb, int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh,
                 int64_t k_ss, int64_t c_sb, int64_t c_ss, void* stream);
-
-/* Measurement aid with no counterpart in the reference: `iters` x 8 v_mfma_f32_32x32x16_bf16 per wave on
- * 256 workgroups of 8 waves, operands taken from `operands` (65536 bf16 values of the caller's choice: the
- * sustained rate depends on the values).  `sink` takes 256 * 512 floats, `clocks` (two 64-bit counters the
- * caller zeroes) accumulates shader-clock and 100 MHz ticks over the workgroups; time the launch with
- * events.  pbs_mfma_probe_flop gives the FLOP count of one launch. */
-int pbs_mfma_probe(const void* operands, int iters, float* sink, unsigned long long* clocks, void* stream);
-double pbs_mfma_probe_flop(int iters);
-
-/* Measurement aid with no counterpart in the reference: the attention kernel's tile pipeline alone.  256
- * workgroups of 8 waves each run `iters` unmasked 128-key tiles for their 256 queries (2 x 128 x 128 block pairs
- * per workgroup and tile, 8.389 MFLOP each) out of LDS, with the kernel's barrier per tile and, if `with_copies`,
- * its asynchronous copies of the next tile (64 KB from a ring of `n_src_tiles` >= 2 K / V^T tile pairs of 65536
- * bytes each at `tiles`, whose first 32 KB also serve as the queries) -- no visit lists, no write-out.  `sink`
- * takes 256 * 512 floats; `clocks` receives workgroup 0's shader-clock ticks and 100 MHz ticks.  Time the launch
- * with events: the same cycles per tile on every input, but on data the clock drops with the power limit. */
-int pbs_attn_tile_probe(const void* tiles, int n_src_tiles, int iters, int with_copies, float* sink,
-                        unsigned long long* clocks, void* stream);
 
 #ifdef __cplusplus
 }

@@ -30,9 +30,6 @@ SIGNATURES = {
     "pbs_sparse_attn_fwd_optional_diagonal": (c_int, [_P] * 9 + [_I] * 6 + [_L] * 9 + [_F, _P, _P]),
     "pbs_unpermute": (c_int, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
     "pbs_rope_qk": (c_int, [_P] * 6 + [_I] * 5 + [_L] * 8 + [_P]),
-    "pbs_mfma_probe": (c_int, [_P, _I, _P, _P, _P]),
-    "pbs_mfma_probe_flop": (ctypes.c_double, [_I]),
-    "pbs_attn_tile_probe": (c_int, [_P, _I, _I, _I, _P, _P, _P]),
     "pbs_identity_indices": (c_int, [_P, _I, _I, _P]),
     "pbs_prefill_attn_workspace_bytes": (_Z, [_I, _I, _I, _I, _I, _I, _I]),
     "pbs_prefill_attn_fwd": (c_int, [_P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I] + [_L] * 12 +

@@ -12,7 +12,10 @@ LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libpbs_hip.so")
 
 SOURCES = ["pbs_abi.hip", "pbs_score.hip", "pbs_sort.hip", "pbs_gather.hip", "pbs_estimate.hip",
-           "pbs_select.hip", "pbs_attn.hip", "pbs_pipeline.hip", "pbs_probe.hip", "pbs_rope.hip"]
+           "pbs_select.hip", "pbs_attn.hip", "pbs_pipeline.hip", "pbs_rope.hip"]
+# measurement kernels for bench.py, in a library of their own: not part of the operator's ABI
+PROBE_SOURCES = ["pbs_probe.hip"]
+PROBE_LIB_PATH = os.path.join(LIB_DIR, "libpbs_probe.so")
 
 DEVICE_FLAGS = ["--offload-arch=gfx950", "-O3", "-fPIC", "-std=c++17",
                 "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
@@ -33,7 +36,7 @@ def build_library(verbose: bool = False) -> str:
     with tempfile.TemporaryDirectory() as tmp:
         objs = []
         procs = []
-        for src in SOURCES:
+        for src in SOURCES + PROBE_SOURCES:
             obj = os.path.join(tmp, src.replace(".hip", ".o"))
             cmd = [hipcc, *DEVICE_FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
             procs.append((src, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True)))
@@ -44,9 +47,14 @@ def build_library(verbose: bool = False) -> str:
                 raise RuntimeError(f"hipcc failed on {src}:\n{err}")
             if verbose and err.strip():
                 print(err)
+        probe_objs = objs[len(SOURCES):]
         tmp_lib = os.path.join(tmp, "libpbs_hip.so")
-        subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp_lib, *objs], check=True)
+        subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp_lib, *objs[:len(SOURCES)]], check=True)
         shutil.move(tmp_lib, LIB_PATH)
+        tmp_probe = os.path.join(tmp, "libpbs_probe.so")
+        subprocess.run([hipcc, "--offload-arch=gfx950", "-shared", "-o", tmp_probe, *probe_objs, "-L" + LIB_DIR, "-lpbs_hip",
+                        "-Wl,-rpath,$ORIGIN"], check=True)
+        shutil.move(tmp_probe, PROBE_LIB_PATH)
     return LIB_PATH
 
 

@@ -34,6 +34,19 @@ int pbs_check_launch(const char* what) {
   return 0;
 }
 
+int pbs_require_no_static_lds(const void* kernel, const char* what) {
+  hipFuncAttributes fa;
+  const hipError_t e = hipFuncGetAttributes(&fa, kernel);
+  if (e != hipSuccess) {
+    pbs_set_error("%s: hipFuncGetAttributes: %s", what, hipGetErrorString(e));
+    return (int)e;
+  }
+  if (fa.sharedSizeBytes != 0)
+    return pbs_arg_error("%s: kernel built with %zu bytes of static LDS; its absolute LDS offsets assume none", what,
+                         (size_t)fa.sharedSizeBytes);
+  return 0;
+}
+
 extern "C" int pbs_abi_version(void) { return 1; }
 
 namespace {

@@ -43,24 +43,11 @@
 //     same pipeline and zeroes the exponentials of keys after the query (key-in-tile > query-in-block).
 //   * careful tiles (a row whose first tile is the diagonal one, and the redo pass): all of S first,
 //     exact running maximum, classic online softmax.
-#include "pbs_common.h"
+#include "pbs_attn_tile.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <atomic>
 
 namespace {
-
-constexpr int D = 128;
-constexpr int BS = 128;
-constexpr int TILE_BYTES = BS * D * 2;            // 32 KB
-constexpr uint32_t LDS_V0 = 2 * TILE_BYTES;       // K buffers at 0 / 32 KB, V buffers at 64 / 96 KB
-constexpr uint32_t LDS_LIST = 4 * TILE_BYTES;     // two merged visit lists (current item, next item), uint16 entries
-constexpr uint32_t LIST_BYTES = 9728;             // count + at most 4096 + 511 + 1 entries, rounded up
-constexpr uint32_t LDS_MISC = LDS_LIST + 2 * LIST_BYTES;   // ints: [1] redo flag, [2] first work item, [4] next work item
-constexpr uint32_t LDS_DUMP = LDS_MISC + 1024;    // 1 KB per wave: landing area of copies issued only to bring lines into L2
-constexpr uint32_t LDS_TOTAL = LDS_DUMP + 8192;   // 159 744 bytes of the CU's 160 KB
-constexpr uint32_t ENT_KB = 0x1fffu;              // visit-list entry: key block ...
-constexpr uint32_t ENT_ORIG = 0x2000u;            // ... | tile of the un-permuted K / V (own segment) | use bits 14, 15
-constexpr int PREFETCH_SLOTS = 2;                 // LDS fragment reads run this many slots ahead
 
 struct AttnArgs {
   const uint16_t* q;
@@ -80,170 +67,7 @@ struct AttnArgs {
   float scale_log2;
 };
 
-typedef __attribute__((address_space(3))) uint8_t lds_u8;
 typedef const __attribute__((address_space(4))) struct AttnArgs* ArgsPtr;
-
-// lane id formed where it is asked for: as a plain intrinsic it is computed once at the top of the kernel and
-// everything derived from it holds registers from there on
-__device__ __forceinline__ int lane_id_here() {
-  int l;
-  asm volatile("v_mbcnt_lo_u32_b32 %0, -1, 0\n\tv_mbcnt_hi_u32_b32 %0, -1, %0" : "=v"(l));
-  return l;
-}
-
-// row of the 32-row MFMA tile -> key of the 32-key sub-tile, chosen so that the accumulator
-// registers 8u..8u+7 of lane-half g hold keys 16u + 8g + 0..7
-__device__ __forceinline__ int mfma_row_to_key(int i) {
-  const int a = i >> 3, g = (i >> 2) & 1, c = i & 3;
-  return 16 * (a >> 1) + 8 * g + 4 * (a & 1) + c;
-}
-
-// ---- asynchronous global -> LDS copy of one 32 KB tile by 512 threads ----------------------
-// global_load_lds_dwordx4 writes lane l at M0 + 16 l, so one wave instruction fills 4 consecutive
-// LDS rows and the chunk swizzle is applied on the GLOBAL side: lane l of wave w fetches chunk
-// (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4).  That chunk does not depend on n: one
-// per-lane byte offset serves the four loads, tile base and LDS base advance by 8192 bytes in
-// scalar registers.  The copy is issued from inline assembly so that the compiler does not order
-// later LDS reads of the OTHER buffer behind it; M0 is handed over as a register operand (the compiler
-// writes it and knows it is in use; the s_nop is the wait state between that write and the copy);
-// completion is awaited with s_waitcnt vmcnt(0) before the barrier that publishes the tile.
-__device__ __forceinline__ uint32_t async_lane_offset(int wave, int lane) {
-  const int row = 4 * wave + (lane >> 4);
-  const int c = (lane & 15) ^ (row & 15);
-  return (uint32_t)((row * D + c * 8) * 2);
-}
-
-__device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t lds_byte, int wave, uint32_t lane_off) {
-  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + wave * 1024));
-  // readfirstlane returns int: widen through uint32_t or the low half would be sign-extended
-  const uint64_t src0 = (uint64_t)(uintptr_t)src;
-  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
-  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
-  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
-#pragma unroll
-  for (int n = 0; n < 4; ++n) {
-    const uint64_t base = srcu + n * 8192;
-    register uint32_t m0v asm("m0") = lds0 + n * 8192;
-    asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(lane_off), "s"(base) : "memory");
-  }
-}
-
-// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride (same LDS layout and swizzle).  Rows
-// past the end of the sequence re-read the last valid row: their keys lie after every query and are masked.
-__device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t row_stride, int rows_valid, uint32_t lds_byte,
-                                                  int wave, int lane) {
-  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + wave * 1024));
-  const uint64_t src0 = (uint64_t)(uintptr_t)src;
-  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
-  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
-  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
-  // lane l of wave w fetches chunk (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4); offsets fit 32 bits
-  // (row stride < 2^22 elements, checked on the host)
-  const uint32_t r0 = (uint32_t)(4 * wave + (lane >> 4));
-  const uint32_t c16 = (uint32_t)(((lane & 15) ^ (r0 & 15)) * 16);
-  if (rows_valid >= BS) {
-    const uint32_t voff = r0 * row_stride * 2u + c16;
-#pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const uint64_t base = srcu + (uint64_t)n * (64u * row_stride);
-      register uint32_t m0v asm("m0") = lds0 + n * 8192;
-      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base) : "memory");
-    }
-  } else {
-#pragma unroll
-    for (int n = 0; n < 4; ++n) {
-      const uint32_t row = min(r0 + 32u * n, (uint32_t)(rows_valid - 1));
-      const uint32_t voff = row * row_stride * 2u + c16;
-      register uint32_t m0v asm("m0") = lds0 + n * 8192;
-      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu) : "memory");
-    }
-  }
-}
-
-__device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
-  return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const lds_u8*)(uintptr_t)byte_addr);
-}
-
-#define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
-
-
-// ---- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved, S of sub-tile s (s <= 3),
-// exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2); S and P are
-// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  The MASKED tile
-// (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
-// query: key-in-tile > query-in-block, an arithmetic test.
-template <bool MASKED, int PF>
-__device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t koff0,
-                                          const uint32_t voff0, const uint32_t (&bx)[8], float c_log2, float& m_ref,
-                                          float& l_part, bool& poisoned, int wq) {
-  // query-in-block minus the lane half's key offset; made opaque per call: the 128 mask compares of a
-  // diagonal tile depend only on the lane, and hoisted out of the tile loop they would each pin a 64-bit
-  // scalar mask
-  int qrel8 = 0;
-  if (MASKED) {
-    const int ln = lane_id_here();          // nothing below may be formed outside the tile
-    qrel8 = 32 * wq + (ln & 31) - 8 * (ln >> 5);
-  }
-  const float negm = -m_ref;
-  float rsum[4] = {0.f, 0.f, 0.f, 0.f};
-  f32x16 sbuf[2];
-  bf16x8 pbuf[2][2];
-  constexpr int R = PF + 1;
-  bf16x8 frk[R], frv[R];
-#pragma unroll
-  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf((koff0 ^ bx[n & 7]) + (n >> 3) * 8192);
-#pragma clang loop unroll(full)
-  for (int n = 0; n < 48; ++n) {
-    const int step = n >> 3, t = n & 7;
-    {   // fragment reads for slot n + PF
-      const int m = n + PF, mstep = m >> 3, mt = m & 7;
-      if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff0 ^ bx[mt]) + mstep * 8192);
-      if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff0 ^ bx[2 * (mstep - 2) + (mt >> 2)]) + (mt & 3) * 8192);
-    }
-    // the reads go out before this slot's matrix instructions: left to the scheduler they sink behind them
-    // (their address is formed in the slot) and the fragments arrive a slot late
-    __builtin_amdgcn_sched_barrier(0);
-    if (step <= 3) {
-      const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
-      sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
-    }
-    if (step >= 2) o[t & 3] = PBS_MFMA(frv[n % R], pbuf[step & 1][t >> 2], o[t & 3]);
-    if (step >= 1 && step <= 4) {
-      const int sb = (step - 1) & 1, r = 2 * t;
-      float x0 = sbuf[sb][r], x1 = sbuf[sb][r + 1];
-      if (MASKED) {
-        // registers r, r + 1 of sub-tile ks hold keys 32 ks + 16 (a4 >> 1) + 8 gh + 4 (a4 & 1) + (r & 3), a4 = r >> 2
-        const int ks = step - 1, a4 = r >> 2;
-        const int key = 32 * ks + 16 * (a4 >> 1) + 4 * (a4 & 1) + (r & 3);
-        if (key > qrel8) x0 = -INFINITY;
-        if (key + 1 > qrel8) x1 = -INFINITY;
-      }
-      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm));
-      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm));
-      rsum[t & 3] += e0;
-      rsum[(t + 2) & 3] += e1;
-      pbuf[sb][r >> 3][r & 7] = (__bf16)e0;
-      pbuf[sb][r >> 3][(r & 7) + 1] = (__bf16)e1;
-    }
-    __builtin_amdgcn_sched_barrier(0);
-  }
-  const float rs = (rsum[0] + rsum[1]) + (rsum[2] + rsum[3]);
-  l_part += rs;
-  // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
-  // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
-  if (__any(rs > 16384.0f)) {
-    const float big = fmaxf(rs, xhalf_f32(rs));
-    if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
-    const float m_new = (big > 16384.0f) ? m_ref + __builtin_amdgcn_logf(big) : m_ref;
-    const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-    m_ref = m_new;
-    l_part *= alpha;
-#pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-  }
-}
 
 // ---- merged visit list of a pair of query blocks, built once per pass by its own kernel:
 // row (bh * npair + pair) of `plist`: [0] = number of tiles, [1 ..] = entries kb | ENT_ORIG? | use_first << 14 |
@@ -318,6 +142,10 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
       int n = total;
       if (own_needed[(int64_t)bh * nb + qb0]) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG | (1u << 14));
       if (second && own_needed[(int64_t)bh * nb + qb1]) out[1 + n++] = (uint16_t)(qb1 | ENT_ORIG | (2u << 14));
+      // a pair that visits nothing still gets one tile (its own block, used by neither query block): the attention
+      // kernel's item protocol -- first tile in flight, claim and hand-over of the next item -- needs no empty case,
+      // and a query block that used no tile writes zeros
+      if (n == 0) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG);
       out[0] = (uint16_t)n;
     }
     return;
@@ -382,13 +210,23 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   int q_begin = a0->xcd_start[xcd], q_end = a0->xcd_start[xcd + 1];   // the range being served: this XCD's, later others'
   int vic = xcd, vic_tried = 0;
   int* misc = reinterpret_cast<int*>(smem + LDS_MISC);   // [1] redo flag, [2] first item, [4] next item
-  if (threadIdx.x == 0) {
-    misc[2] = q_begin + atomicAdd(a0->queue + xcd, 1);
-    misc[1] = 0;
+  // the first item: from this XCD's range, or, when that one is empty or already handed out, from the next XCD's
+  // range that still has items
+  int cur;
+  for (;;) {
+    if (threadIdx.x == 0) {
+      misc[2] = q_begin + atomicAdd(a0->queue + vic, 1);
+      misc[1] = 0;
+    }
+    __syncthreads();
+    cur = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[2]), a0->interleave, npair);
+    if (cur < q_end) break;
+    if (++vic_tried > 7) return;
+    vic = (xcd + vic_tried) & 7;
+    q_begin = a0->xcd_start[vic];
+    q_end = a0->xcd_start[vic + 1];
+    __syncthreads();   // everyone has read the ticket before the next one is written
   }
-  __syncthreads();
-  int cur = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[2]), a0->interleave, npair);
-  if (cur >= q_end) return;
   int nxt = q_end;   // the next item is claimed late in the current one: an item claimed early waits for this
                      // workgroup while others may be idle
   bool has_nxt = false;
@@ -658,7 +496,10 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       // ---- epilogue: normalise, transpose through LDS (same swizzle), coalesced 16-byte stores.  The staging
       // area is the pair of buffers the last tile sat in (the other pair is receiving the next item's first
       // tile): its K buffer for the first query block, its V buffer for the second.
-      const float inv = 1.0f / (l_part + xhalf_f32(l_part));
+      // a query block that used no tile (no selected block and no own block: possible only with an optional diagonal)
+      // has a zero sum and writes zeros, as the reference does for a row without selected blocks
+      const float l_all = l_part + xhalf_f32(l_part);
+      const float inv = l_all == 0.f ? 0.f : 1.0f / l_all;
       // lane-dependent addresses of the epilogue come from a fresh opaque lane id: derived from the item's one
       // they would be computed at the top of the item and held across the tile loop
       const int lane_e = lane_id_here();
@@ -734,68 +575,6 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     nxt = q_end;
     has_nxt = false;
     if (wave == 0 && lane_id_here() == 0) misc[1] = 0;   // read by everyone before the epilogue's barrier, set again only after the next item's barriers
-  }
-}
-
-// ---- measurement aid: the tile pipeline alone.  Every workgroup runs `iters` unmasked fast tiles out of its two
-// LDS buffer pairs with the kernel's per-tile barrier and, if asked, the kernel's 64 KB of copies per tile (from a
-// ring of `n_src` K / V^T tile pairs), without lists, items, write-out or rare paths: what the schedule of
-// fast_tile sustains by itself.  Workgroup 0 reports its shader-clock and 100 MHz ticks.
-__global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __restrict__ tiles, int n_src, int iters, int with_copies,
-                                                            float* __restrict__ sink, unsigned long long* __restrict__ clocks) {
-  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
-  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
-  for (int i = threadIdx.x; i < (int)(4 * TILE_BYTES / 16); i += 512)   // both buffer pairs start as copies of the first tiles
-    reinterpret_cast<u32x4*>(smem)[i] = reinterpret_cast<const u32x4*>(tiles)[i % (2 * TILE_BYTES / 16)];
-  __syncthreads();
-  const int lane = lane_id_here();
-  const int j = lane & 31, gh = lane >> 5;
-  const int krow = mfma_row_to_key(j);
-  const uint32_t koff0 = (uint32_t)(krow * 256 + ((gh ^ (krow & 15)) * 16));
-  const uint32_t voff0 = LDS_V0 + (uint32_t)(j * 256 + ((gh ^ (j & 15)) * 16));
-  const uint32_t lane_off = async_lane_offset(wave, lane);
-  bf16x8 qf[8];
-#pragma unroll
-  for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(tiles + (wave * 32 + j) * D + 16 * t + 8 * gh);
-  f32x16 o[4];
-  float zero = 0.f;
-  asm volatile("" : "+v"(zero));
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) o[dt][r] = zero;
-  float m_ref = 8.f, l_part = 0.f, c_log2 = 0.12751743f;   // exp2(s / sqrt(128) * log2 e - 8): no rescale on N(0, 1) data
-  asm volatile("" : "+s"(c_log2));
-  bool poisoned = false;
-  uint32_t bufx = 0;
-  const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
-  for (int it = 0; it < iters; ++it, bufx ^= 0x8000u) {
-    __builtin_amdgcn_s_waitcnt(0x0f70);
-    __syncthreads();
-    if (with_copies) {
-      const uint16_t* src = tiles + (size_t)((it * 7 + (int)blockIdx.x / 8) % n_src) * (2 * BS * D);
-      stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off);
-      stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
-    }
-    uint32_t bx[8];
-#pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      bx[t] = bufx ^ (uint32_t)(t << 5);
-      asm volatile("" : "+s"(bx[t]));
-    }
-    fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wave & 3);
-  }
-  __builtin_amdgcn_s_waitcnt(0x0f70);
-  const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
-  float s = l_part + m_ref + (poisoned ? 1.f : 0.f);
-#pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
-#pragma unroll
-    for (int r = 0; r < 16; ++r) s += o[dt][r];
-  sink[blockIdx.x * 512 + threadIdx.x] = s;
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    clocks[0] = c1 - c0;
-    clocks[1] = r1 - r0;
   }
 }
 
@@ -916,6 +695,7 @@ static int sparse_attn_launch(const void* q, const void* perm_k, const void* per
   // fewer when there are fewer items
   const int64_t n_wg = std::min<int64_t>((int64_t)8 * max_items, (int64_t)(n_cu + 7) / 8 * 8);
   if (attr == hipSuccess && !(tracked && (g_lds_reserved.load(std::memory_order_acquire) >> dev & 1))) {
+    if (const int rc = pbs_require_no_static_lds((const void*)sparse_attn_kernel, "pbs_sparse_attn_fwd")) return rc;
     attr = hipFuncSetAttribute((const void*)sparse_attn_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
     if (attr == hipSuccess && tracked) g_lds_reserved.fetch_or(1ull << dev, std::memory_order_release);
   }
@@ -927,18 +707,4 @@ static int sparse_attn_launch(const void* q, const void* perm_k, const void* per
                      (uint16_t*)((char*)workspace + 256), a.queue, a.nb, a.bps, a.cap, own_block_needed);
   hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(512), LDS_TOTAL, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_sparse_attn_fwd");
-}
-
-extern "C" int pbs_attn_tile_probe(const void* tiles, int n_src_tiles, int iters, int with_copies, float* sink,
-                                   unsigned long long* clocks, void* stream) {
-  PBS_REQUIRE(tiles && sink && clocks && iters > 0 && n_src_tiles >= 2, "pbs_attn_tile_probe: bad arguments");
-  PBS_REQUIRE(((uintptr_t)tiles % 16) == 0, "pbs_attn_tile_probe: tiles must be 16-byte aligned");
-  hipError_t attr = hipFuncSetAttribute((const void*)tile_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
-  if (attr != hipSuccess) {
-    pbs_set_error("pbs_attn_tile_probe: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
-    return (int)attr;
-  }
-  hipLaunchKernelGGL(tile_probe_kernel, dim3(256), dim3(512), LDS_TOTAL, (hipStream_t)stream, (const uint16_t*)tiles, n_src_tiles,
-                     iters, with_copies, sink, clocks);
-  return pbs_check_launch("pbs_attn_tile_probe");
 }

@@ -19,6 +19,10 @@ extern "C" const char* pbs_last_error(void);
 void pbs_set_error(const char* fmt, ...);
 int pbs_arg_error(const char* fmt, ...);        // sets message, returns -1
 int pbs_check_launch(const char* what);         // hipGetLastError -> positive code
+// Kernels that address LDS by absolute byte offsets (M0 of global_load_lds, integer-to-LDS-pointer casts) rely on
+// their dynamic LDS starting at offset 0, i.e. on having no static LDS: 0 if `kernel` has none, else an error code
+// with the message set.
+int pbs_require_no_static_lds(const void* kernel, const char* what);
 
 #define PBS_REQUIRE(cond, ...)                      \
   do {                                              \

@@ -42,6 +42,15 @@ Layout make_layout(int B, int Hq, int Hkv, int S, int D, int block_size, int seg
   return L;
 }
 
+// A sequence that fits inside one segment is plain causal attention (pbs_attn/src/pbs.py:175-182): identity key
+// order, every causal block visited.  With that order and every candidate selected the result does not depend on the
+// segment size, so the kernels run with one segment spanning the sequence or, beyond the attention kernel's 511
+// blocks per segment, with segments of 256 blocks.  Returns the segment size to run with.
+int one_segment_size(int S, int block_size) {
+  const int nb = (S + block_size - 1) / block_size;
+  return (nb <= 511 ? nb : 256) * block_size;
+}
+
 }  // namespace
 
 extern "C" int pbs_identity_indices(int32_t* key_indices, int rows, int S_pad, void* stream) {
@@ -54,7 +63,7 @@ extern "C" int pbs_identity_indices(int32_t* key_indices, int rows, int S_pad, v
 
 extern "C" size_t pbs_prefill_attn_workspace_bytes(int B, int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size) {
   if (B <= 0 || Hq <= 0 || Hkv <= 0 || Hq % Hkv || S <= 0 || head_dim <= 0 || block_size <= 0 || segment_size <= 0) return 0;
-  if (S <= segment_size) segment_size = (S + block_size - 1) / block_size * block_size;   // as pbs_prefill_attn_fwd
+  if (S <= segment_size) segment_size = one_segment_size(S, block_size);   // as pbs_prefill_attn_fwd
   return make_layout(B, Hq, Hkv, S, head_dim, block_size, segment_size).total;
 }
 
@@ -71,14 +80,15 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
               "pbs_prefill_attn_fwd: segment_size must be a multiple of block_size");
   // sequences that fit one segment: plain causal attention = one segment spanning the sequence,
   // identity order, every causal block visited
-  if (S <= segment_size) {
-    segment_size = (S + block_size - 1) / block_size * block_size;
+  const bool one_segment = S <= segment_size;
+  if (one_segment) {
+    segment_size = one_segment_size(S, block_size);
     threshold_is_int_one = 1;
   }
   // checked here, before anything is enqueued (the attention kernel holds one segment's blocks in its list)
   PBS_REQUIRE(segment_size / block_size <= 511,
-              "pbs_prefill_attn_fwd: a segment of %d blocks exceeds the limit of 511 (a sequence that fits inside "
-              "one segment may be at most 65408 tokens; use a smaller segment_size)", segment_size / block_size);
+              "pbs_prefill_attn_fwd: a segment of %d blocks exceeds the limit of 511 (use a smaller segment_size)",
+              segment_size / block_size);
   const Layout L = make_layout(B, Hq, Hkv, S, head_dim, block_size, segment_size);
   PBS_REQUIRE(workspace && workspace_bytes >= L.total, "pbs_prefill_attn_fwd: workspace too small (%zu < %zu bytes)",
               workspace_bytes, L.total);
@@ -87,7 +97,7 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
   const int rows = B * Hq, nb = (S + block_size - 1) / block_size, s_pad = nb * block_size;
   const int nseg = S / segment_size, rem = S % segment_size;
   int rc;
-  if (nseg == 0 || (nseg == 1 && rem == 0)) {
+  if (one_segment || nseg == 0 || (nseg == 1 && rem == 0)) {
     if ((rc = pbs_identity_indices((int32_t*)(w + L.idx), rows, s_pad, stream))) return rc;
   } else {
     if ((rc = pbs_score_keys(q, k, (float*)(w + L.scores), B, Hq, Hkv, S, head_dim, block_size, segment_size, q_sb, q_sh,

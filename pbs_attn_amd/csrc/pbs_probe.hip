@@ -3,8 +3,8 @@
 // (zeros run at the full clock, normally distributed values make the chip lower its clock to stay inside
 // its power limit), so the benchmark reports it next to the attention kernel's rate as the MFMA ceiling
 // for data like the attention kernel's.
-#include "pbs_common.h"
-#include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
+#include "pbs_attn_tile.h"
+#include "pbs_probe.h"   // the definitions below are checked against these declarations
 
 namespace {
 
@@ -46,4 +46,84 @@ extern "C" int pbs_mfma_probe(const void* operands, int iters, float* sink, unsi
 
 extern "C" double pbs_mfma_probe_flop(int iters) {
   return (double)PROBE_WGS * (PROBE_THREADS / 64) * (double)iters * 8.0 * (2.0 * 32 * 32 * 16);
+}
+
+namespace {
+
+// ---- measurement aid: the tile pipeline alone.  Every workgroup runs `iters` unmasked fast tiles out of its two
+// LDS buffer pairs with the kernel's per-tile barrier and, if asked, the kernel's 64 KB of copies per tile (from a
+// ring of `n_src` K / V^T tile pairs), without lists, items, write-out or rare paths: what the schedule of
+// fast_tile sustains by itself.  Workgroup 0 reports its shader-clock and 100 MHz ticks.
+__global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __restrict__ tiles, int n_src, int iters, int with_copies,
+                                                            float* __restrict__ sink, unsigned long long* __restrict__ clocks) {
+  extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+  const int wave = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  for (int i = threadIdx.x; i < (int)(4 * TILE_BYTES / 16); i += 512)   // both buffer pairs start as copies of the first tiles
+    reinterpret_cast<u32x4*>(smem)[i] = reinterpret_cast<const u32x4*>(tiles)[i % (2 * TILE_BYTES / 16)];
+  __syncthreads();
+  const int lane = lane_id_here();
+  const int j = lane & 31, gh = lane >> 5;
+  const int krow = mfma_row_to_key(j);
+  const uint32_t koff0 = (uint32_t)(krow * 256 + ((gh ^ (krow & 15)) * 16));
+  const uint32_t voff0 = LDS_V0 + (uint32_t)(j * 256 + ((gh ^ (j & 15)) * 16));
+  const uint32_t lane_off = async_lane_offset(wave, lane);
+  bf16x8 qf[8];
+#pragma unroll
+  for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(tiles + (wave * 32 + j) * D + 16 * t + 8 * gh);
+  f32x16 o[4];
+  float zero = 0.f;
+  asm volatile("" : "+v"(zero));
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[dt][r] = zero;
+  float m_ref = 8.f, l_part = 0.f, c_log2 = 0.12751743f;   // exp2(s / sqrt(128) * log2 e - 8): no rescale on N(0, 1) data
+  asm volatile("" : "+s"(c_log2));
+  bool poisoned = false;
+  uint32_t bufx = 0;
+  const unsigned long long c0 = __builtin_amdgcn_s_memtime(), r0 = __builtin_amdgcn_s_memrealtime();
+  for (int it = 0; it < iters; ++it, bufx ^= 0x8000u) {
+    __builtin_amdgcn_s_waitcnt(0x0f70);
+    __syncthreads();
+    if (with_copies) {
+      const uint16_t* src = tiles + (size_t)((it * 7 + (int)blockIdx.x / 8) % n_src) * (2 * BS * D);
+      stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off);
+      stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+    }
+    uint32_t bx[8];
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      bx[t] = bufx ^ (uint32_t)(t << 5);
+      asm volatile("" : "+s"(bx[t]));
+    }
+    fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wave & 3);
+  }
+  __builtin_amdgcn_s_waitcnt(0x0f70);
+  const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
+  float s = l_part + m_ref + (poisoned ? 1.f : 0.f);
+#pragma unroll
+  for (int dt = 0; dt < 4; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += o[dt][r];
+  sink[blockIdx.x * 512 + threadIdx.x] = s;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    clocks[0] = c1 - c0;
+    clocks[1] = r1 - r0;
+  }
+}
+
+}  // namespace
+
+extern "C" int pbs_attn_tile_probe(const void* tiles, int n_src_tiles, int iters, int with_copies, float* sink,
+                                   unsigned long long* clocks, void* stream) {
+  PBS_REQUIRE(tiles && sink && clocks && iters > 0 && n_src_tiles >= 2, "pbs_attn_tile_probe: bad arguments");
+  PBS_REQUIRE(((uintptr_t)tiles % 16) == 0, "pbs_attn_tile_probe: tiles must be 16-byte aligned");
+  hipError_t attr = hipFuncSetAttribute((const void*)tile_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
+  if (attr != hipSuccess) {
+    pbs_set_error("pbs_attn_tile_probe: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
+    return (int)attr;
+  }
+  hipLaunchKernelGGL(tile_probe_kernel, dim3(256), dim3(512), LDS_TOTAL, (hipStream_t)stream, (const uint16_t*)tiles, n_src_tiles,
+                     iters, with_copies, sink, clocks);
+  return pbs_check_launch("pbs_attn_tile_probe");
 }

@@ -10,6 +10,7 @@
 // divide: fp32 accumulate -> bf16 -> / sqrt(D) -> bf16.
 #include "pbs_common.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
+#include <atomic>
 #include <mutex>
 
 namespace {
@@ -280,6 +281,12 @@ int score_keys_launch(const char* who, const void* q, const void* k, float* scor
   a.part = (float*)workspace;
   a.stats = a.part + (size_t)B * Hq * a.nchunk * NQ * 2;
   a.scores = scores;
+  static std::atomic<bool> lds_checked{false};   // once per process: a property of the code object
+  if (!lds_checked.load(std::memory_order_acquire)) {
+    if (const int rc = pbs_require_no_static_lds((const void*)score_kernel<false>, who)) return rc;
+    if (const int rc = pbs_require_no_static_lds((const void*)score_kernel<true>, who)) return rc;
+    lds_checked.store(true, std::memory_order_release);
+  }
   hipStream_t st = (hipStream_t)stream;
   dim3 grid(a.nchunk, B * Hkv);
   const dim3 block(Hq / Hkv > 1 ? 256 : 64);

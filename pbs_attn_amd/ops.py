@@ -278,11 +278,10 @@ def prefill_attn_fwd(q, k, v, block_size, segment_size, threshold, force_select_
     if softmax_scale is None:
         softmax_scale = 1.0 / math.sqrt(D)
     is_int_one, thr_rows, thr = _threshold_args(threshold, B, Hq, q.device)
-    seg_blocks = (S + block_size - 1) // block_size if S <= segment_size else segment_size // block_size
-    if seg_blocks > 511:
+    if S > segment_size and segment_size // block_size > 511:
         raise _lib.PbsHipError(
-            f"a segment of {seg_blocks} blocks exceeds the attention kernel's limit of 511 (a sequence that fits "
-            f"inside one segment may be at most 65408 tokens): use a smaller segment_size")
+            f"a segment of {segment_size // block_size} blocks exceeds the attention kernel's limit of 511: "
+            f"use a smaller segment_size")
     out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
     ws_bytes = lib.pbs_prefill_attn_workspace_bytes(B, Hq, Hkv, S, D, block_size, segment_size)
     ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=q.device)

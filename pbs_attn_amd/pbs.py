@@ -69,14 +69,14 @@ def _identity_indices(B, H, s_pad, device):
 
 
 def apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode="mean",
-                      scores: Optional[torch.Tensor] = None) -> PermutedKV:
+                      scores: Optional[torch.Tensor] = None, identity: bool = False) -> PermutedKV:
     """Permutation phase (pbs.py:185-190 + :213-215): score keys with the last query
     block, sort inside each segment, gather K and V.  ``scores`` can be injected
-    to run the sort on a given score tensor."""
+    to run the sort on a given score tensor; ``identity`` keeps the keys in their order."""
     B, Hq, S, D = query_states.shape
     nseg, rem = S // segment_size, S % segment_size
     s_pad = (S + block_size - 1) // block_size * block_size
-    if nseg == 0 or (nseg == 1 and rem == 0):               # permute_states.py:36-38
+    if identity or nseg == 0 or (nseg == 1 and rem == 0):               # permute_states.py:36-38
         idx = _identity_indices(B, Hq, s_pad, query_states.device)
     else:
         if scores is None:
@@ -178,15 +178,19 @@ def permuted_block_sparse_attn_fwd(
         return ops.prefill_attn_fwd(query_states, key_states, value_states, block_size, segment_size, threshold,
                                     force_select_first_block, query_pool_mode, key_pool_mode)
 
-    if q_len <= segment_size:
-        # pbs.py:175-182: plain causal attention.  Same kernel, one segment spanning the
-        # sequence, identity order, every causal block visited.
-        segment_size = (q_len + block_size - 1) // block_size * block_size
+    one_segment = q_len <= segment_size
+    if one_segment:
+        # pbs.py:175-182: plain causal attention.  Same kernel, identity order, every causal block visited: one
+        # segment spanning the sequence or, beyond the kernel's 511 blocks per segment, segments of 256 blocks
+        # (with that order and everything selected the result does not depend on the segment size).
+        nb = (q_len + block_size - 1) // block_size
+        segment_size = (nb if nb <= 511 else 256) * block_size
         threshold = 1
 
     if isinstance(threshold, int) and threshold == 1:
         # every candidate is selected: no estimate, one full gather
-        perm = apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode)
+        perm = apply_permutation(query_states, key_states, value_states, block_size, segment_size, key_pool_mode,
+                                 identity=one_segment)
         sel = permuted_block_selection(query_states, perm, block_size, segment_size, threshold, causal,
                                        force_select_first_block, query_pool_mode, key_pool_mode, want_masks=False)
     else:

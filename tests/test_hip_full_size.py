@@ -194,6 +194,27 @@ def test_sequence_inside_one_large_segment_is_plain_causal_attention(dev):
     assert_attn_close(out, _sdpa(q, k, v), what="S <= segment_size vs SDPA")
 
 
+def test_long_sequence_inside_one_larger_segment_is_plain_causal_attention(dev):
+    # S <= segment_size beyond the 511 blocks one segment of the attention kernel may hold (782 blocks here):
+    # identity order and everything selected give the same result with any segment size, so the path runs with
+    # segments of 256 blocks; single call and staged path, both against SDPA
+    S = 100000
+    q, k, v = make_qkv(1, 2, 1, S, 128, "uniform_heavy", seed=14, device=dev)
+    ref = _sdpa(q, k, v)
+    out = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 131072, 0.9, True)
+    assert_attn_close(out, ref, what="S = 100000 <= segment_size vs SDPA")
+
+    class Null:
+        def mark(self, name):
+            pass
+    P.stage_timer = Null()
+    try:
+        staged = P.permuted_block_sparse_attn_fwd(q, k, v, 128, 131072, 0.9, True)
+    finally:
+        P.stage_timer = None
+    assert torch.equal(out, staged)
+
+
 def test_longest_supported_sequence(dev):
     # 4096 blocks (524 283 tokens, ragged): the limits of the visit list, the long-row selection kernel and
     # the split of two heads over eight XCDs; sampled rows against dense fp32 attention on the path's own mask

@@ -121,3 +121,39 @@ def test_stage_adapters_with_the_reference_signatures(dev):
     P = compat.block_pooled_attn(qd, perm_k, 128, cand.to(dev))
     assert torch.allclose(P.cpu()[~nan], ref_scores[~nan], rtol=3e-2, atol=1e-6)
     assert torch.equal(compat.first_token_mask(idx, 128).cpu(), O.first_token_mask(idx.cpu(), 128))
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,S,thr", [(1, 4, 2, 2048, 1.5), (2, 2, 2, 1000, 1.0), (1, 3, 1, 1536, 1.0), (1, 2, 2, 128, 2.0),
+                                            (1, 1, 1, 4096, 1.5)])
+def test_query_blocks_that_select_nothing_give_zeros(dev, B, Hq, Hkv, S, thr):
+    """force_select_first_block=False and force_select_current_block=False with a threshold the running sum never
+    reaches (above 1, or 1.0 against a float32 sum that tops out below it): select_blocks picks nothing for such a
+    row (utils.py:74-84) and the attention gives zeros for it (kernels/...:340-343).  Whole launches without a single
+    tile, pairs of query blocks where one or both visit nothing, and rows that do reach the threshold, side by side."""
+    q, k, v = small_case(B, Hq, Hkv, S, seed=S + Hq + 5)
+    ke, ve = expand_kv(q, k), expand_kv(q, v)
+    ref_out, mid = O.meanpooling_prefill(q, ke, ve, 128, 1024, thr, True, False, False, return_intermediates=True)
+    empty_rows = ~mid["block_mask"].any(-1)
+    assert empty_rows.any(), "the case is meant to leave query blocks without a block"
+    if thr > 1.0:
+        assert empty_rows.all() and (ref_out == 0).all()
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    nb = (S + 127) // 128
+    idx = torch.arange(nb * 128, dtype=torch.int32, device=dev).view(1, 1, -1).expand(B, Hq, -1).contiguous()
+    sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, False, candidate_rule=2)
+    assert torch.equal(sel.cpu(), mid["block_mask"])
+    own = sel.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    out = torch.full_like(qd, float("nan"))
+    ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=own, out=out)
+    out = out.cpu()
+    dense = torch.nan_to_num(O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128), nan=0.0)
+    assert_attn_close(out, dense, what="rows without blocks: HIP vs dense fp32 (zeros where nothing is selected)")
+    row_empty = empty_rows.repeat_interleave(128, -1)[..., :S]
+    assert (out[row_empty] == 0).all()
+    # the whole mode from raw Q, K, V, twice (the second call finds the first one's lists in the workspace)
+    for _ in range(2):
+        out2, got = MeanPooling_prefill(qd, kd, vd, 128, 1024, thr, True, False, False, return_masks=True)
+        own_mask = got["block_mask"].cpu()
+        dense2 = torch.nan_to_num(O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], own_mask, 128), nan=0.0)
+        assert_attn_close(out2.cpu(), dense2, what="MeanPooling_prefill with unreachable threshold vs dense fp32 on its own mask")

@@ -31,6 +31,34 @@ def test_patched_model_matches_unpatched_on_gpu(dev, name):
     assert torch.isfinite(lg.float()).all()
 
 
+def test_llama31_8b_prompt_of_65536_tokens(dev):
+    """BASELINE.json's config 4 at its own prompt length (65 536 uniform random token ids, the Llama-3.1-8B
+    architecture with random weights; two of the 32 identical layers): patched with every causal block selected
+    the model must reproduce the unpatched one on the logits of the last 256 positions; patched with the default
+    threshold (which drops a tenth of the estimated attention mass) it must stay finite; the distance is printed."""
+    from pbs_attn.patch.huggingface import apply_patch_with_prefill, get_permuted_block_sparse_attn_fwd
+    from pbs_attn_amd.ttft import build_model
+    model = build_model("llama31_8b", layers=2, device=dev)
+    ids = torch.randint(0, 128256, (1, 65536), generator=torch.Generator().manual_seed(4)).to(dev)
+    with torch.no_grad():
+        ref = model(ids, logits_to_keep=256).logits.float()
+        assert ref.shape == (1, 256, 128256)
+        apply_patch_with_prefill(model, get_permuted_block_sparse_attn_fwd(segment_size=256, threshold=1))
+        got = model(ids, logits_to_keep=256).logits.float()
+        d = (got - ref).abs()
+        print(f"\n64k prompt, threshold=1 against the unpatched model: max {d.max():.4f} mean {d.mean():.5f}")
+        assert d.max() < 0.15 and d.mean() < 0.02, (d.max(), d.mean())
+        for layer in model.model.layers:            # patch again with the factory's defaults (threshold 0.9)
+            layer.self_attn.forward = layer.self_attn.original_forward
+        apply_patch_with_prefill(model, get_permuted_block_sparse_attn_fwd())
+        sparse = model(ids, logits_to_keep=256).logits.float()
+        assert torch.isfinite(sparse).all()
+        d = (sparse - ref).abs()
+        print(f"64k prompt, threshold=0.9 against the unpatched model: max {d.max():.4f} mean {d.mean():.5f}")
+        out = model.generate(ids, max_new_tokens=1, do_sample=False)
+        assert out.shape == (1, 65537)
+
+
 @pytest.mark.parametrize("method", ["pbs", "meanpooling", "dense"])
 def test_ttft_harness_writes_the_reference_result_record(dev, method, tmp_path, capsys):
     """The offline harness follows eval/efficiency/eval_efficiency.py: one JSON line on stdout and a result

@@ -463,8 +463,8 @@ def test_rope_qk_bitwise_equals_the_tensor_expression(dev, B, Hq, Hkv, S, cos_ba
 
 
 def test_mfma_probe_runs_and_counts_clocks(dev):
-    from pbs_attn_amd import _lib
-    lib = _lib.load()
+    import bench
+    lib = bench.load_probe_library()   # the benchmark's measurement kernels live in a library of their own
     pool = torch.randn(65536, device=dev).bfloat16()
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     clocks = torch.zeros(2, dtype=torch.int64, device=dev)

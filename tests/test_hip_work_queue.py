@@ -70,8 +70,9 @@ def test_work_distribution_shapes_against_dense_attention_on_the_mask(dev, B, Hq
 
 def test_tile_pipeline_probe_runs_and_reports_clocks(dev):
     """The measurement entry point: a short run on zero and on random tiles returns finite sums and both clock counters."""
+    import bench
     from pbs_attn_amd import _lib
-    lib = _lib.load()
+    lib = bench.load_probe_library()
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     st = torch.cuda.current_stream().cuda_stream
     for ring in (torch.zeros(4 * 32768, dtype=torch.bfloat16, device=dev),
