@@ -14,9 +14,11 @@ step time).  A second, untimed-for-`value` pass runs the same work stage by stag
 a HIP event after every stage: `stage_ms`, and `roofline`, which prices the dominant
 kernel (the block-sparse attention) against the bf16 dense MFMA peak.  `cpu_baseline`
 times the CPU restatement of the reference's torch path on a bounded sample on this
-host's cores.  The default run adds two more measurements as extra keys: `cfg1` (the
-32k layer: segment 256, threshold 0.9) and `ttft_llama31_8b_64k` (time to first token
-of the 32-layer architecture on a 64k prompt, patched against unpatched).
+host's cores.  The default run adds the other configurations as extra keys: `cfg0` (4k), `cfg1`
+(the 32k layer: segment 256, threshold 0.9), `cfg1_sweep` (threshold x segment size at 32k), `cfg3`
+(the batched 7:1 layer), `permutation_ablation` (PBS against the un-permuted MeanPooling mode) and
+`ttft_llama31_8b_64k` (time to first token of the 32-layer architecture on a 64k prompt, patched
+against unpatched).
 """
 from __future__ import annotations
 
@@ -304,10 +306,12 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     kv_once = B * Hkv * S * D * e                       # one of K, V at the KV heads
     score_b = kv_once + B * Hq * bs * D * e + B * Hq * S * 4
     pool_b = kv_once + B * Hq * S * 4 + 2 * B * Hq * nb * D * e + B * Hq * S * D * e    # K, indices, Q in; pooled out
-    # reads: the K and V rows of the gathered blocks (each row counted once per KV head at most), their indices,
-    # V again for the original-order transposed copy; writes: the gathered tiles and that copy
-    gather_b = (2 * min(f * B * Hq, B * Hkv) * S * D * e + f * B * Hq * S * 4 + kv_once
-                + 2 * f * B * Hq * S * D * e + kv_once)
+    # reads: the K and V rows of the gathered blocks (each row counted once per KV head at most) and their indices;
+    # writes: the gathered tiles.  The original-order transposed copy of V that the same launch writes for the
+    # attention kernel's own-segment tiles (V read once more, the copy written) is this design's own extra traffic
+    # and is reported beside the rate, not in it.
+    gather_b = 2 * min(f * B * Hq, B * Hkv) * S * D * e + f * B * Hq * S * 4 + 2 * f * B * Hq * S * D * e
+    res["gather_extra_bytes_orig_vt"] = 2 * kv_once
     est_b = (0 if "pool" in stages else B * Hq * S * D * e) + 2 * B * Hq * nb * D * e + B * Hq * nb * nb * 4
     res["hbm_gbs"] = {
         "score": score_b / (stages["score"] * 1e-3) / 1e9 if "score" in stages else None,
@@ -365,6 +369,41 @@ def meanpooling_mode(torch, cfg, q, k, v, reps=2):
     e1.record()
     torch.cuda.synchronize()
     return pairs / (B * Hq * nb * (nb + 1) // 2), e0.elapsed_time(e1) / reps
+
+
+def side_summary(torch, name, overrides, steps, warmup, with_dense=True):
+    """One more configuration measured like the headline one, condensed to the figures of a table row."""
+    r, inputs = run_workload(torch, name, steps, warmup, overrides=overrides, with_dense=with_dense, min_warm_ms=150.0)
+    del inputs
+    torch.cuda.empty_cache()
+    log(f"[bench] {name} {overrides} " + json.dumps(r))
+    a = r["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / (r["stage_ms"]["sparse_attn"] * 1e-3) / 1e12
+    out = {"workload": f"{name}: B={r['B']} Hq={r['Hq']} Hkv={r['Hkv']} S={r['S']}, block {r['block']}, segment {r['segment']}, "
+                       f"threshold {r['threshold']}, generator {r['generator']} seed {r['seed']}",
+           "segment": r["segment"], "threshold": r["threshold"],
+           "ms_per_step": r["ms_per_step"], "value": r["effective_tflops_pipeline"], "unit": "TFLOP/s",
+           "density_vs_causal": r["density_vs_causal"], "stage_ms": r["stage_ms"],
+           "attn_kernel_tflops": a, "attn_kernel_frac_of_peak": a / PEAK_BF16_TFLOPS}
+    if with_dense:
+        out.update(dense_sdpa_ms=r.get("dense_sdpa_ms"), dense_own_kernel_ms=r.get("dense_own_kernel_ms"),
+                   speedup_vs_dense_sdpa=r.get("speedup_vs_dense_sdpa"))
+    return out
+
+
+def ablation(torch, name, overrides, res):
+    """PBS (permuted) against MeanPooling_prefill (the same estimate and selection without the permutation) on one
+    input: block density of the two masks and the time of one pass each."""
+    from pbs_attn_amd.synth import make_workload
+    if res is None:
+        res, (cfg, q, k, v) = run_workload(torch, name, 3, 2, overrides=overrides, with_dense=False)
+    else:
+        cfg, q, k, v = make_workload(name, seed=0, device=torch.device("cuda:0"), **overrides)
+    mp_density, mp_ms = meanpooling_mode(torch, cfg, q, k, v)
+    del q, k, v
+    torch.cuda.empty_cache()
+    return {"workload": f"{name}: S={cfg['S']}, segment {cfg['segment']}, threshold {cfg['threshold']}, generator {cfg['kind']}",
+            "pbs_density": res["density_vs_causal"], "pbs_ms": res["ms_per_step"],
+            "meanpooling_density": mp_density, "meanpooling_ms": mp_ms}
 
 
 def ttft_pair(torch, length=65536, runs=3, warmup=1, model_name="llama31_8b", layers=None):
@@ -436,7 +475,7 @@ def main():
     ap.add_argument("--no-mfma-probe", action="store_true", help="skip the MFMA-only ceiling measurement")
     ap.add_argument("--cpu-seconds", type=float, default=20.0)
     ap.add_argument("--no-extras", action="store_true",
-                    help="skip the two extra measurements of the default run (the 32k layer and the 64k time to first token)")
+                    help="skip the extra measurements of the default run (the other configurations, the ablation, the 64k time to first token)")
     ap.add_argument("--report", default=None, metavar="FILE.md",
                     help="run every single-layer configuration and the sweeps, write a markdown table, and exit")
     ap.add_argument("--traffic-calibration", action="store_true",
@@ -502,6 +541,7 @@ def main():
         "ms_per_step_staged": res["ms_per_step_staged"],
         "hbm_gbs": res["hbm_gbs"],
         "gathered_block_fraction": res["gathered_block_fraction"],
+        "gather_extra_bytes_orig_vt": res["gather_extra_bytes_orig_vt"],
         "dense_sdpa_ms": res.get("dense_sdpa_ms"),
         "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
         "speedup_vs_dense_sdpa": res.get("speedup_vs_dense_sdpa"),
@@ -519,19 +559,18 @@ def main():
     del inputs
     torch.cuda.empty_cache()
     if not (args.no_extras or overrides or args.workload != "cfg2"):
-        # the other two figures the headline metric names, measured the same way in the same run
-        r1, inputs1 = run_workload(torch, "cfg1", max(args.steps, 10), max(args.warmup, 3), min_warm_ms=150.0)
-        del inputs1
-        torch.cuda.empty_cache()
-        log("[bench] cfg1 " + json.dumps(r1))
-        a1 = r1["visited_block_pairs"] * FLOP_PER_BLOCK_PAIR / (r1["stage_ms"]["sparse_attn"] * 1e-3) / 1e12
-        line["cfg1"] = {
-            "workload": f"cfg1: same layer shape, S={r1['S']}, block {r1['block']}, segment {r1['segment']}, threshold "
-                        f"{r1['threshold']}, generator {r1['generator']} seed {r1['seed']}",
-            "ms_per_step": r1["ms_per_step"], "value": r1["effective_tflops_pipeline"], "unit": "TFLOP/s",
-            "density_vs_causal": r1["density_vs_causal"], "stage_ms": r1["stage_ms"],
-            "attn_kernel_tflops": a1, "attn_kernel_frac_of_peak": a1 / PEAK_BF16_TFLOPS,
-            "dense_sdpa_ms": r1.get("dense_sdpa_ms"), "speedup_vs_dense_sdpa": r1.get("speedup_vs_dense_sdpa")}
+        # the other figures the headline metric names and the other configurations, measured the same way in the same run
+        line["cfg1"] = side_summary(torch, "cfg1", {}, steps=max(args.steps, 10), warmup=max(args.warmup, 3))
+        line["cfg0"] = side_summary(torch, "cfg0", {}, steps=20, warmup=5)
+        line["cfg3"] = side_summary(torch, "cfg3", {}, steps=10, warmup=3)
+        # config 1's sweep: threshold x segment size on the 32k layer (the dense baseline is the one of `cfg1`)
+        line["cfg1_sweep"] = [side_summary(torch, "cfg1", {"threshold": th, "segment": sg}, steps=5, warmup=2, with_dense=False)
+                              for sg in (256, 1024) for th in (0.8, 0.9, 0.95)]
+        # the sparse regime: the headline shape on an input whose attention has the structure PBS exploits
+        line["cfg2_strong_heavy"] = side_summary(torch, "cfg2", {"kind": "strong_heavy"}, steps=10, warmup=3, with_dense=False)
+        # what the permutation buys: PBS against the reference's un-permuted MeanPooling baseline (same block size
+        # and threshold through the same kernels) on the headline input and on one whose heavy keys are scattered
+        line["permutation_ablation"] = [ablation(torch, "cfg2", {}, res), ablation(torch, "cfg2", {"kind": "strong_uniform"}, None)]
         line["ttft_llama31_8b_64k"] = ttft_pair(torch)
         log("[bench] ttft " + json.dumps(line["ttft_llama31_8b_64k"]))
     print(json.dumps(line), flush=True)
