@@ -254,10 +254,12 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
   auto stage_entry = [&](const HeadBase& hb, uint32_t e, uint32_t buf, int lane, uint32_t lane_off) {
     const int kb_e = (int)(e & ENT_KB);
     if (e & ENT_ORIG) {
-      stage_krows_async(hb.korig + (int64_t)kb_e * BS * hb.k_ss, hb.k_ss, hb.S - kb_e * BS, buf, wave, lane);
+      // the lane id is formed afresh: offsets derived from the item's one are loop invariants that get hoisted out of
+      // the tile loop and, when registers run out there, spilled and reloaded per tile
+      stage_krows_async(hb.korig + (int64_t)kb_e * BS * hb.k_ss, hb.k_ss, hb.S - kb_e * BS, buf, wave, lane_id_here());
       stage_tile_async(hb.ovt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
     } else {
-      stage_tile_async(hb.pk + (int64_t)kb_e * BS * D, buf, wave, lane_off);
+      stage_tile_async(hb.pk + (int64_t)kb_e * BS * D, buf, wave, lane_off ^ k_copy_xor(wave));
       stage_tile_async(hb.pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
     }
   };
@@ -285,16 +287,22 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     // everything per lane is derived afresh from the lane id in every item: nothing but scalars lives across items
     const int lane = lane_id_here();
     const int tid = wave * 64 + lane;
-    const int j = lane & 31, gh = lane >> 5;
+    const int i16 = lane & 15, g4 = lane >> 4;
     // per-lane LDS byte offsets of the fragments inside buffer 0; XOR 0x8000 switches buffer.
-    //   K fragment (sub-tile ks, d-step t)      : koff[t] + ks * 8192
-    //   V fragment (keys 16 c .. 16 c + 15, dt) : voff[c] + dt * 8192
-    // The 16-byte chunk index is XORed with the row: fragment t of a row lies at (offset of fragment 0) ^ (t << 5),
-    // so one per-lane offset per operand serves all eight; the XOR constant is merged with the buffer switch in
-    // scalar registers (bx[] below), one vector XOR per read either way.
-    const int krow = mfma_row_to_key(j);
-    const uint32_t koff0 = (uint32_t)(krow * 256 + ((gh ^ (krow & 15)) * 16));
-    const uint32_t voff0 = LDS_V0 + (uint32_t)(j * 256 + ((gh ^ (j & 15)) * 16));
+    //   K fragment (sub-tile ks, row tile T, d-step kd) : (koff0 ^ kd << 6) + T * 1024 + ks * 8192
+    //   V^T fragment (sub-tile ks, d tile dt)           : (voff0 ^ ks << 6) + dt * 4096
+    // The 16-byte chunk index is XORed with a hash of the row, so the fragments of a row lie at (offset of the
+    // first) ^ (n << 6).
+    const int krow = 8 * (i16 >> 2) + (i16 & 3);   // k_row_hash(krow) == i16
+    const uint32_t koff0 = (uint32_t)(krow * 256 + ((g4 ^ i16) * 16));
+    const uint32_t voff0 = LDS_V0 + (uint32_t)(i16 * 256 + ((g4 ^ i16) * 16));
+    // the addresses in the buffers of the item's first tile; switched to the other buffers after every tile
+    uint32_t ka[4], va[4];
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      ka[n] = koff0 ^ (uint32_t)(n << 6) ^ par;
+      va[n] = voff0 ^ (uint32_t)(n << 6) ^ par;
+    }
     const uint32_t lane_off = async_lane_offset(wave, lane);
     int claim = 0;   // ticket of the next item: in flight during one tile
 
@@ -305,15 +313,16 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     const int qb = 2 * pair + grp;
     const bool qb_valid = qb < ap->nb;
     const float c_log2 = ap->scale_log2;
-    const int qpos = qb * BS + 32 * wq + j;
+    const int qpos = qb * BS + 32 * wq + i16;
 
-    // Q^T fragments (B operand): query column j, d = 16 t + 8 gh + 0..7.  Rows past the end of the sequence
-    // compute on the last row's values and are never stored.
-    bf16x8 qf[8];
-    {
-      const uint16_t* qrow = ap->q + b * ap->q_sb + h * ap->q_sh + (int64_t)min(qpos, ap->S - 1) * ap->q_ss;
+    // Q^T fragments (B operand): query column 16 qg + i16, d = 32 kd + 8 g4 + 0..7.  Rows past the end of the
+    // sequence compute on the last row's values and are never stored.
+    bf16x8 qf[2][4];
 #pragma unroll
-      for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(qrow + 16 * t + 8 * gh);
+    for (int qg = 0; qg < 2; ++qg) {
+      const uint16_t* qrow = ap->q + b * ap->q_sb + h * ap->q_sh + (int64_t)min(qpos + 16 * qg, ap->S - 1) * ap->q_ss;
+#pragma unroll
+      for (int kd = 0; kd < 4; ++kd) qf[qg][kd] = *reinterpret_cast<const bf16x8*>(qrow + 32 * kd + 8 * g4);
     }
     const int n_tiles = __builtin_amdgcn_readfirstlane((int)mlist[0]);
     // the next item: claimed three tiles before the end of this one (the counter's latency passes under a
@@ -352,17 +361,19 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     };
 
     {
-      f32x16 o[4];
+      f32x4 o[8][2];   // [d tile][query column group]
       {
-        float zero = 0.f;   // opaque: a constant zero vector would be kept (and spilled) as sixteen registers
+        float zero = 0.f;   // opaque: a constant zero vector would be kept (and spilled) as registers of its own
         asm volatile("" : "+v"(zero));
 #pragma unroll
-        for (int dt = 0; dt < 4; ++dt)
+        for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) o[dt][r] = zero;
+          for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) o[dt][qg][r] = zero;
       }
-      float m_ref = -INFINITY;   // reference maximum, identical in lanes j and j + 32
-      float l_part = 0.f;        // row sum of this lane's half of the keys
+      float m_ref[2] = {-INFINITY, -INFINITY};   // reference maxima of queries i16 and 16 + i16, identical in the four lanes i16 + 16 g
+      float l_part[2] = {0.f, 0.f};              // row sums over this lane's quarter of the keys
       bool first = true, poisoned = false;
       bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
 
@@ -374,7 +385,15 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1]), par, lane, lane_off);
       }
       uint32_t bufx = par;
-      for (int it = 0; it < n_tiles; ++it, bufx ^= 0x8000u) {
+      auto next_buffers = [&]() {
+        bufx ^= 0x8000u;
+#pragma unroll
+        for (int n = 0; n < 4; ++n) {
+          ka[n] ^= 0x8000u;
+          va[n] ^= 0x8000u;
+        }
+      };
+      for (int it = 0; it < n_tiles; ++it, next_buffers()) {
         const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
         const int kb = (int)(ent & ENT_KB);
         __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` (and of the next list) has landed
@@ -386,12 +405,6 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         else if (has_nxt && (careful_only || n_tiles >= 3))   // shorter items: after the loop, once the list has landed
           stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx ^ 0x8000u, lane, lane_off);
         if (!(ent & use_bit) || !qb_valid) continue;
-        uint32_t bx[8];   // buffer switch ^ fragment index << 5: opaque, or the compiler folds the constant into eight per-lane offsets
-#pragma unroll
-        for (int t = 0; t < 8; ++t) {
-          bx[t] = bufx ^ (uint32_t)(t << 5);
-          asm volatile("" : "+s"(bx[t]));
-        }
         const bool masked = (ent & ENT_ORIG) && kb == qb;   // the diagonal block; other own-segment blocks lie before it
 
         // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
@@ -400,78 +413,92 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
           // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good
           // enough reference to start the pipelined path (later keys move it up lazily)
           first = false;
-          f32x16 s0 = (f32x16){0};
+          float mx[2] = {-INFINITY, -INFINITY};
 #pragma unroll
-          for (int t = 0; t < 8; ++t) s0 = PBS_MFMA(ldsf(koff0 ^ bx[t]), qf[t], s0);
-          float mx = s0[0];
+          for (int T = 0; T < 2; ++T) {
+            f32x4 s0[2] = {(f32x4){0}, (f32x4){0}};
 #pragma unroll
-          for (int r = 1; r < 16; ++r) mx = fmaxf(mx, s0[r]);
-          mx = fmaxf(mx, xhalf_f32(mx));
-          m_ref = mx * c_log2;
+            for (int kd = 0; kd < 4; ++kd) {
+              const bf16x8 fk = ldsf(ka[kd] + T * 1024);
+#pragma unroll
+              for (int qg = 0; qg < 2; ++qg) s0[qg] = PBS_MFMA(fk, qf[qg][kd], s0[qg]);
+            }
+#pragma unroll
+            for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+              for (int r = 0; r < 4; ++r) mx[qg] = fmaxf(mx[qg], s0[qg][r]);
+          }
+#pragma unroll
+          for (int qg = 0; qg < 2; ++qg) m_ref[qg] = max_over_lane_groups(mx[qg]) * c_log2;
           all_seen = true;
-          fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
+          fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
         } else if (first || careful_only || (masked && !all_seen)) {
-          // ---------------- careful tile
+          // ---------------- careful tile: classic online softmax, one 32-key sub-tile at a time
           first = false;
-          f32x16 s[4];
+#pragma nounroll
+          for (int ks = 0; ks < 4; ++ks) {   // a real loop: the rare path stays small, in code and in registers
+            f32x4 s[2][2];   // [T][qg]
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks) {
-            s[ks] = (f32x16){0};
+            for (int T = 0; T < 2; ++T) {
+              s[T][0] = (f32x4){0};
+              s[T][1] = (f32x4){0};
 #pragma unroll
-            for (int t = 0; t < 8; ++t) s[ks] = PBS_MFMA(ldsf((koff0 ^ bx[t]) + ks * 8192), qf[t], s[ks]);
-          }
-          if (masked) {
-            const int ln = lane_id_here();   // keep the compares inside the tile (see fast_tile)
-            const int qrel = 32 * wq + (ln & 31), gh = ln >> 5;
+              for (int kd = 0; kd < 4; ++kd) {
+                const bf16x8 fk = ldsf(ka[kd] + T * 1024 + ks * 8192);
 #pragma unroll
-            for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int a4 = r >> 2;
-                const int key = 32 * ks + 16 * (a4 >> 1) + 8 * gh + 4 * (a4 & 1) + (r & 3);
-                if (key > qrel) s[ks][r] = -INFINITY;
+                for (int qg = 0; qg < 2; ++qg) s[T][qg] = PBS_MFMA(fk, qf[qg][kd], s[T][qg]);
               }
-          }
-          float mx = -INFINITY;
-#pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s[ks][r]);
-          mx = fmaxf(mx, xhalf_f32(mx));
-          const float m_new = fmaxf(m_ref, mx * c_log2);
-          const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-          const float alpha = __builtin_amdgcn_exp2f(m_ref - m_use);
-          float rs = 0.f;
-#pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float p = __builtin_amdgcn_exp2f(s[ks][r] * c_log2 - m_use);
-              s[ks][r] = p;
-              rs += p;
             }
-          l_part = l_part * alpha + rs;
-          m_ref = m_new;
-          all_seen = !__any(m_ref == -INFINITY);
-          if (__any(alpha != 1.0f)) {
+            if (masked) {
+              const int ln = lane_id_here();   // keep the compares inside the tile (see fast_tile)
+              const int qrel8 = 32 * wq + (ln & 15) - 8 * (ln >> 4);
 #pragma unroll
-            for (int dt = 0; dt < 4; ++dt)
+              for (int T = 0; T < 2; ++T)
 #pragma unroll
-              for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
-          }
+                for (int qg = 0; qg < 2; ++qg)
 #pragma unroll
-          for (int ks = 0; ks < 4; ++ks)
-#pragma unroll
-            for (int u = 0; u < 2; ++u) {
-              bf16x8 pf;
-#pragma unroll
-              for (int e = 0; e < 8; ++e) pf[e] = (__bf16)s[ks][8 * u + e];
-#pragma unroll
-              for (int dt = 0; dt < 4; ++dt) o[dt] = PBS_MFMA(ldsf((voff0 ^ bx[2 * ks + u]) + dt * 8192), pf, o[dt]);
+                  for (int r = 0; r < 4; ++r)
+                    if (32 * ks + 4 * T + r - 16 * qg > qrel8) s[T][qg][r] = -INFINITY;
             }
+            float alpha[2];
+            bf16x8 pf[2];
+#pragma unroll
+            for (int qg = 0; qg < 2; ++qg) {
+              float mx = fmaxf(fmaxf(s[0][qg][0], s[0][qg][1]), fmaxf(s[0][qg][2], s[0][qg][3]));
+              mx = fmaxf(mx, fmaxf(fmaxf(s[1][qg][0], s[1][qg][1]), fmaxf(s[1][qg][2], s[1][qg][3])));
+              mx = max_over_lane_groups(mx);
+              const float m_new = fmaxf(m_ref[qg], mx * c_log2);
+              const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+              alpha[qg] = __builtin_amdgcn_exp2f(m_ref[qg] - m_use);
+              m_ref[qg] = m_new;
+              float rs = 0.f;
+#pragma unroll
+              for (int e = 0; e < 8; ++e) {
+                const float pe = __builtin_amdgcn_exp2f(s[e >> 2][qg][e & 3] * c_log2 - m_use);
+                rs += pe;
+                pf[qg][e] = (__bf16)pe;
+              }
+              l_part[qg] = l_part[qg] * alpha[qg] + rs;
+            }
+            if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
+#pragma unroll
+              for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+                for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) o[dt][qg][r] *= alpha[qg];
+            }
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) {
+              const bf16x8 fv = ldsf((va[0] ^ (uint32_t)(ks << 6)) + dt * 4096);
+#pragma unroll
+              for (int qg = 0; qg < 2; ++qg) o[dt][qg] = PBS_MFMA(fv, pf[qg], o[dt][qg]);
+            }
+          }
+          all_seen = !__any(m_ref[0] == -INFINITY || m_ref[1] == -INFINITY);
         } else {
-          if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
-          else fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wq);
+          if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+          else fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
         }
       }
       if (!careful_only && n_tiles < 3) {
@@ -498,24 +525,28 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       // tile): its K buffer for the first query block, its V buffer for the second.
       // a query block that used no tile (no selected block and no own block: possible only with an optional diagonal)
       // has a zero sum and writes zeros, as the reference does for a row without selected blocks
-      const float l_all = l_part + xhalf_f32(l_part);
-      const float inv = l_all == 0.f ? 0.f : 1.0f / l_all;
+      float inv[2];
+#pragma unroll
+      for (int qg = 0; qg < 2; ++qg) {
+        const float l_all = sum_over_lane_groups(l_part[qg]);
+        inv[qg] = l_all == 0.f ? 0.f : 1.0f / l_all;
+      }
       // lane-dependent addresses of the epilogue come from a fresh opaque lane id: derived from the item's one
       // they would be computed at the top of the item and held across the tile loop
       const int lane_e = lane_id_here();
-      const int j_e = lane_e & 31, gh_e = lane_e >> 5;
+      const int i_e = lane_e & 15, g_e = lane_e >> 4;
       const uint32_t last_buf = par ^ (((n_tiles - 1) & 1) ? 0x8000u : 0u);
       uint16_t* os = reinterpret_cast<uint16_t*>(smem + last_buf + (grp ? LDS_V0 : 0u));
 #pragma unroll
-      for (int dt = 0; dt < 4; ++dt)
+      for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-          const int row = 32 * wq + j_e;
-          const int c = 4 * dt + a4;   // 16-byte chunk of d = 32 dt + 8 a4 + 4 gh + 0..3
+        for (int qg = 0; qg < 2; ++qg) {
+          const int row = 32 * wq + 16 * qg + i_e;
+          const int c = 2 * dt + (g_e >> 1);   // 16-byte chunk of d = 16 dt + 4 g + 0..3
           bf16x4 v4;
 #pragma unroll
-          for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][4 * a4 + cc] * inv);
-          *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * gh_e) = v4;
+          for (int cc = 0; cc < 4; ++cc) v4[cc] = (__bf16)(o[dt][qg][cc] * inv[qg]);
+          *reinterpret_cast<bf16x4*>(os + row * D + ((c ^ (row & 15)) * 8) + 4 * (g_e & 1)) = v4;
         }
       __syncthreads();
       if (qb_valid) {

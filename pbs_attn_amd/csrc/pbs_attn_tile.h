@@ -30,17 +30,28 @@ __device__ __forceinline__ int lane_id_here() {
   return l;
 }
 
-// row of the 32-row MFMA tile -> key of the 32-key sub-tile, chosen so that the accumulator
-// registers 8u..8u+7 of lane-half g hold keys 16u + 8g + 0..7
-__device__ __forceinline__ int mfma_row_to_key(int i) {
-  const int a = i >> 3, g = (i >> 2) & 1, c = i & 3;
-  return 16 * (a >> 1) + 8 * g + 4 * (a & 1) + c;
-}
+// ---- operand geometry of a wave (32 queries = two column groups qg of 16; lane l: i = l % 16, g = l / 16)
+//   S^T = K Q^T per 32-key sub-tile ks: two 16-key row tiles T, four d-steps kd of 32:
+//       A = K[key(T, i)][32 kd + 8 g + 0..7],  key(T, i) = 32 ks + 8 (i / 4) + 4 T + i % 4
+//       B = Q[16 qg + i][32 kd + 8 g + 0..7]
+//       D: lane holds query 16 qg + i, keys 32 ks + 8 g + 4 T + 0..3
+//     so the eight values of (T = 0, T = 1) are keys 32 ks + 8 g + 0..7: converted to bf16 they ARE the B operand of
+//   O^T += V^T P^T per sub-tile: eight 16-row d tiles dt:
+//       A = V^T[16 dt + i][32 ks + 8 g + 0..7],  B = P[keys 32 ks + 8 g + 0..7][16 qg + i]
+//       D: lane holds query 16 qg + i, d = 16 dt + 4 g + 0..3
+// LDS tiles are 128 rows x 16 chunks of 16 bytes, chunk index XOR hash(row): rows of a K tile are keys and the 16
+// lanes of a fragment read take keys 8 (i / 4) + i % 4 (+ 4 T), so the hash is (row & 3) | ((row >> 3) & 3) << 2
+// (= i: sixteen chunks, no bank conflict); rows of a V^T tile are d and the lanes take consecutive rows: row & 15.
+__device__ __forceinline__ int k_row_hash(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
+
+// the copy of a K tile fetches chunk (l & 15) ^ k_row_hash(row) where async_lane_offset has (l & 15) ^ (row & 15), row =
+// 4 wave + (l >> 4) + 32 n: the two differ by a wave-uniform XOR of the byte offset
+__device__ __forceinline__ uint32_t k_copy_xor(int wave) { return (uint32_t)(((wave & 3) ^ ((wave >> 1) & 3)) << 6); }
 
 // ---- asynchronous global -> LDS copy of one 32 KB tile by 512 threads ----------------------
 // global_load_lds_dwordx4 writes lane l at M0 + 16 l, so one wave instruction fills 4 consecutive
 // LDS rows and the chunk swizzle is applied on the GLOBAL side: lane l of wave w fetches chunk
-// (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4).  That chunk does not depend on n: one
+// (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4) (a V^T tile; for a K tile the offset is XORed with k_copy_xor).  That chunk does not depend on n: one
 // per-lane byte offset serves the four loads, tile base and LDS base advance by 8192 bytes in
 // scalar registers.  The copy is issued from inline assembly so that the compiler does not order
 // later LDS reads of the OTHER buffer behind it; M0 is handed over as a register operand (the compiler
@@ -67,7 +78,7 @@ __device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t l
   }
 }
 
-// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride (same LDS layout and swizzle).  Rows
+// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride (the LDS layout of a K tile, k_row_hash below).  Rows
 // past the end of the sequence re-read the last valid row: their keys lie after every query and are masked.
 __device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t row_stride, int rows_valid, uint32_t lds_byte,
                                                   int wave, int lane) {
@@ -79,7 +90,7 @@ __device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t 
   // lane l of wave w fetches chunk (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4); offsets fit 32 bits
   // (row stride < 2^22 elements, checked on the host)
   const uint32_t r0 = (uint32_t)(4 * wave + (lane >> 4));
-  const uint32_t c16 = (uint32_t)(((lane & 15) ^ (r0 & 15)) * 16);
+  const uint32_t c16 = (uint32_t)(((lane & 15) ^ k_row_hash((int)r0)) * 16);
   if (rows_valid >= BS) {
     const uint32_t voff = r0 * row_stride * 2u + c16;
 #pragma unroll
@@ -103,84 +114,113 @@ __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
   return *reinterpret_cast<const __attribute__((address_space(3))) bf16x8*>((const lds_u8*)(uintptr_t)byte_addr);
 }
 
-#define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0)
+// v_mfma_f32_16x16x32_bf16: D (16 x 16) += A (16 x 32) B (32 x 16).  Lane l holds row l % 16 of A and column l % 16 of
+// B, each with k = 8 (l / 16) + 0..7, and of D column l % 16, rows 4 (l / 16) + 0..3.  On normally distributed
+// operands the chip sustains about 11 % more FLOP/s with this shape than with 32x32x16 (it moves half the
+// accumulator registers per FLOP and holds a higher clock inside its power limit).
+#define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
 
+// lane ^ 16: with xhalf_f32 (lane ^ 32) it reaches the four lanes that share a query column
+__device__ __forceinline__ float xq16_f32(float v) { return __shfl_xor(v, 16, 64); }
+__device__ __forceinline__ float max_over_lane_groups(float v) {
+  v = fmaxf(v, xq16_f32(v));
+  return fmaxf(v, xhalf_f32(v));
+}
+__device__ __forceinline__ float sum_over_lane_groups(float v) {
+  v += xq16_f32(v);
+  return v + xhalf_f32(v);
+}
 
 // ---- fast tile: 48 slots = 6 steps x 8.  Step s issues, interleaved, S of sub-tile s (s <= 3),
 // exponentials of sub-tile s - 1 (1 <= s <= 4), P.V of sub-tile s - 2 (s >= 2); S and P are
-// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  The MASKED tile
-// (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
+// double-buffered by sub-tile parity; one scheduling barrier per slot keeps the order.  A slot reads one K and one
+// V^T fragment (two slots ahead) and feeds each to two matrix instructions, one per query column group.  The MASKED
+// tile (the diagonal block, read in original key order) zeroes the exponentials of keys that lie after the
 // query: key-in-tile > query-in-block, an arithmetic test.
+// ka[kd] / va[ks]: this lane's byte addresses of the K fragments of d-step kd (row tile 0, sub-tile 0) and of the V^T
+// fragments of sub-tile ks (d tile 0) in the tile's buffers: held in registers and switched between the two buffers
+// once per tile, so that a fragment read needs no address arithmetic (a vector instruction per read is a tenth of
+// the pipeline's vector work, and vector work overlaps only a third of a matrix instruction's time).
 template <bool MASKED, int PF>
-__device__ __forceinline__ void fast_tile(f32x16 (&o)[4], const bf16x8 (&qf)[8], const uint32_t koff0,
-                                          const uint32_t voff0, const uint32_t (&bx)[8], float c_log2, float& m_ref,
-                                          float& l_part, bool& poisoned, int wq) {
-  // query-in-block minus the lane half's key offset; made opaque per call: the 128 mask compares of a
+__device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2][4], const uint32_t (&ka)[4],
+                                          const uint32_t (&va)[4], float c_log2, float (&m_ref)[2],
+                                          float (&l_part)[2], bool& poisoned, int wq) {
+  // query-in-block minus the lane group's key offset; made opaque per call: the mask compares of a
   // diagonal tile depend only on the lane, and hoisted out of the tile loop they would each pin a 64-bit
   // scalar mask
   int qrel8 = 0;
   if (MASKED) {
     const int ln = lane_id_here();          // nothing below may be formed outside the tile
-    qrel8 = 32 * wq + (ln & 31) - 8 * (ln >> 5);
+    qrel8 = 32 * wq + (ln & 15) - 8 * (ln >> 4);
   }
-  const float negm = -m_ref;
-  float rsum[4] = {0.f, 0.f, 0.f, 0.f};
-  f32x16 sbuf[2];
-  bf16x8 pbuf[2][2];
+  const float negm[2] = {-m_ref[0], -m_ref[1]};
+  float rsum[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  f32x4 sacc[2][2][2];     // [sub-tile parity][T][qg]
+  bf16x8 pbuf[2][2];       // [sub-tile parity][qg]
   constexpr int R = PF + 1;
   bf16x8 frk[R], frv[R];
 #pragma unroll
-  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf((koff0 ^ bx[n & 7]) + (n >> 3) * 8192);
+  for (int n = 0; n < PF; ++n) frk[n % R] = ldsf(ka[n & 3] + ((n >> 2) & 1) * 1024 + (n >> 3) * 8192);
 #pragma clang loop unroll(full)
   for (int n = 0; n < 48; ++n) {
     const int step = n >> 3, t = n & 7;
     {   // fragment reads for slot n + PF
       const int m = n + PF, mstep = m >> 3, mt = m & 7;
-      if (m < 48 && mstep <= 3) frk[m % R] = ldsf((koff0 ^ bx[mt]) + mstep * 8192);
-      if (m < 48 && mstep >= 2) frv[m % R] = ldsf((voff0 ^ bx[2 * (mstep - 2) + (mt >> 2)]) + (mt & 3) * 8192);
+      if (m < 48 && mstep <= 3) frk[m % R] = ldsf(ka[mt & 3] + (mt >> 2) * 1024 + mstep * 8192);
+      if (m < 48 && mstep >= 2) frv[m % R] = ldsf(va[mstep - 2] + mt * 4096);
     }
     // the reads go out before this slot's matrix instructions: left to the scheduler they sink behind them
     // (their address is formed in the slot) and the fragments arrive a slot late
     __builtin_amdgcn_sched_barrier(0);
     if (step <= 3) {
-      const f32x16 acc = (t == 0) ? (f32x16){0} : sbuf[step & 1];
-      sbuf[step & 1] = PBS_MFMA(frk[n % R], qf[t], acc);
+      const int T = t >> 2, kd = t & 3;
+#pragma unroll
+      for (int qg = 0; qg < 2; ++qg) {
+        const f32x4 acc = (kd == 0) ? (f32x4){0} : sacc[step & 1][T][qg];
+        sacc[step & 1][T][qg] = PBS_MFMA(frk[n % R], qf[qg][kd], acc);
+      }
     }
-    if (step >= 2) o[t & 3] = PBS_MFMA(frv[n % R], pbuf[step & 1][t >> 2], o[t & 3]);
+    if (step >= 2) {
+#pragma unroll
+      for (int qg = 0; qg < 2; ++qg) o[t][qg] = PBS_MFMA(frv[n % R], pbuf[step & 1][qg], o[t][qg]);
+    }
     if (step >= 1 && step <= 4) {
-      const int sb = (step - 1) & 1, r = 2 * t;
-      float x0 = sbuf[sb][r], x1 = sbuf[sb][r + 1];
+      const int sb = (step - 1) & 1, qg = t >> 2, T = (t >> 1) & 1, c0 = 2 * (t & 1);
+      float x0 = sacc[sb][T][qg][c0], x1 = sacc[sb][T][qg][c0 + 1];
       if (MASKED) {
-        // registers r, r + 1 of sub-tile ks hold keys 32 ks + 16 (a4 >> 1) + 8 gh + 4 (a4 & 1) + (r & 3), a4 = r >> 2
-        const int ks = step - 1, a4 = r >> 2;
-        const int key = 32 * ks + 16 * (a4 >> 1) + 4 * (a4 & 1) + (r & 3);
+        // the two values are keys 32 ks + 8 g + 4 T + c0 (+ 1) of query 32 wq + 16 qg + i
+        const int key = 32 * (step - 1) + 4 * T + c0 - 16 * qg;
         if (key > qrel8) x0 = -INFINITY;
         if (key + 1 > qrel8) x1 = -INFINITY;
       }
-      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm));
-      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm));
-      rsum[t & 3] += e0;
-      rsum[(t + 2) & 3] += e1;
-      pbuf[sb][r >> 3][r & 7] = (__bf16)e0;
-      pbuf[sb][r >> 3][(r & 7) + 1] = (__bf16)e1;
+      const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm[qg]));
+      const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm[qg]));
+      rsum[qg][0] += e0;
+      rsum[qg][1] += e1;
+      pbuf[sb][qg][4 * T + c0] = (__bf16)e0;
+      pbuf[sb][qg][4 * T + c0 + 1] = (__bf16)e1;
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  const float rs = (rsum[0] + rsum[1]) + (rsum[2] + rsum[3]);
-  l_part += rs;
+  const float rs[2] = {rsum[0][0] + rsum[0][1], rsum[1][0] + rsum[1][1]};
+  l_part[0] += rs[0];
+  l_part[1] += rs[1];
   // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
   // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
-  if (__any(rs > 16384.0f)) {
-    const float big = fmaxf(rs, xhalf_f32(rs));
-    if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
-    const float m_new = (big > 16384.0f) ? m_ref + __builtin_amdgcn_logf(big) : m_ref;
-    const float alpha = __builtin_amdgcn_exp2f(m_ref - m_new);
-    m_ref = m_new;
-    l_part *= alpha;
+  if (__any(rs[0] > 16384.0f || rs[1] > 16384.0f)) {
 #pragma unroll
-    for (int dt = 0; dt < 4; ++dt)
+    for (int qg = 0; qg < 2; ++qg) {
+      const float big = max_over_lane_groups(rs[qg]);
+      if (__any(!(big < 1e30f))) poisoned = true;   // overflow (inf / nan): redo the row without speculation
+      const float m_new = (big > 16384.0f) ? m_ref[qg] + __builtin_amdgcn_logf(big) : m_ref[qg];
+      const float alpha = __builtin_amdgcn_exp2f(m_ref[qg] - m_new);
+      m_ref[qg] = m_new;
+      l_part[qg] *= alpha;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) o[dt][r] *= alpha;
+      for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[dt][qg][r] *= alpha;
+    }
   }
 }
 

@@ -62,22 +62,27 @@ __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __re
     reinterpret_cast<u32x4*>(smem)[i] = reinterpret_cast<const u32x4*>(tiles)[i % (2 * TILE_BYTES / 16)];
   __syncthreads();
   const int lane = lane_id_here();
-  const int j = lane & 31, gh = lane >> 5;
-  const int krow = mfma_row_to_key(j);
-  const uint32_t koff0 = (uint32_t)(krow * 256 + ((gh ^ (krow & 15)) * 16));
-  const uint32_t voff0 = LDS_V0 + (uint32_t)(j * 256 + ((gh ^ (j & 15)) * 16));
+  const int i16 = lane & 15, g4 = lane >> 4;
+  const int krow = 8 * (i16 >> 2) + (i16 & 3);
+  const uint32_t koff0 = (uint32_t)(krow * 256 + ((g4 ^ i16) * 16));
+  const uint32_t voff0 = LDS_V0 + (uint32_t)(i16 * 256 + ((g4 ^ i16) * 16));
   const uint32_t lane_off = async_lane_offset(wave, lane);
-  bf16x8 qf[8];
+  bf16x8 qf[2][4];
 #pragma unroll
-  for (int t = 0; t < 8; ++t) qf[t] = *reinterpret_cast<const bf16x8*>(tiles + (wave * 32 + j) * D + 16 * t + 8 * gh);
-  f32x16 o[4];
+  for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+    for (int kd = 0; kd < 4; ++kd)
+      qf[qg][kd] = *reinterpret_cast<const bf16x8*>(tiles + (wave * 32 + 16 * qg + i16) * D + 32 * kd + 8 * g4);
+  f32x4 o[8][2];
   float zero = 0.f;
   asm volatile("" : "+v"(zero));
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
+  for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) o[dt][r] = zero;
-  float m_ref = 8.f, l_part = 0.f, c_log2 = 0.12751743f;   // exp2(s / sqrt(128) * log2 e - 8): no rescale on N(0, 1) data
+    for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) o[dt][qg][r] = zero;
+  float m_ref[2] = {8.f, 8.f}, l_part[2] = {0.f, 0.f}, c_log2 = 0.12751743f;   // exp2(s / sqrt(128) * log2 e - 8): no rescale on N(0, 1) data
   asm volatile("" : "+s"(c_log2));
   bool poisoned = false;
   uint32_t bufx = 0;
@@ -87,24 +92,26 @@ __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __re
     __syncthreads();
     if (with_copies) {
       const uint16_t* src = tiles + (size_t)((it * 7 + (int)blockIdx.x / 8) % n_src) * (2 * BS * D);
-      stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off);
+      stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off ^ k_copy_xor(wave));
       stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
     }
-    uint32_t bx[8];
+    uint32_t ka[4], va[4];
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      bx[t] = bufx ^ (uint32_t)(t << 5);
-      asm volatile("" : "+s"(bx[t]));
+    for (int n = 0; n < 4; ++n) {
+      ka[n] = koff0 ^ (uint32_t)(n << 6) ^ bufx;
+      va[n] = voff0 ^ (uint32_t)(n << 6) ^ bufx;
     }
-    fast_tile<false, PREFETCH_SLOTS>(o, qf, koff0, voff0, bx, c_log2, m_ref, l_part, poisoned, wave & 3);
+    fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wave & 3);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);
   const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
-  float s = l_part + m_ref + (poisoned ? 1.f : 0.f);
+  float s = l_part[0] + l_part[1] + m_ref[0] + m_ref[1] + (poisoned ? 1.f : 0.f);
 #pragma unroll
-  for (int dt = 0; dt < 4; ++dt)
+  for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) s += o[dt][r];
+    for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) s += o[dt][qg][r];
   sink[blockIdx.x * 512 + threadIdx.x] = s;
   if (blockIdx.x == 0 && threadIdx.x == 0) {
     clocks[0] = c1 - c0;
