@@ -211,8 +211,9 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
 
 // ---------------------------------------------------------------------------------------------
 // Wave-level variant (rows of up to 1024 blocks): ONE wave per row, the row lives in registers.
-//   * bitonic network on 64-bit composite keys, NPL keys per lane: strides below NPL are register
-//     compare-exchanges, larger strides exchange with lane ^ (stride / NPL); no barriers;
+//   * bitonic network on the 32-bit value keys, NPL keys per lane: strides below NPL are register
+//     compare-exchanges, larger strides exchange with lane ^ (stride / NPL); no barriers; the stable order's
+//     tie-break by index is applied only where it matters, at the value where the threshold is reached;
 //   * the running sum is first taken as a parallel float64 prefix (local prefixes + wave scan).  It
 //     differs from the sequential sum by < 1e-12, so "float32(prefix) >= threshold" is decided from it
 //     unless some prefix up to the first hit lies within 1e-11 of the float32 rounding boundary of the
@@ -220,8 +221,9 @@ __global__ __launch_bounds__(256) void select_blocks_kernel(SelectArgs a) {
 //     decision is the one the sequential float64 sum gives;
 //   * flags, own-segment minima, masks and the compacted visit list as in the block-level kernel.
 // ---------------------------------------------------------------------------------------------
+// The bitonic network on 32-bit keys, NPL per lane: a compare-exchange is a minimum and a maximum.
 template <int NPL>
-__device__ __forceinline__ void wave_bitonic_sort(uint64_t (&k)[NPL], int lane) {
+__device__ __forceinline__ void wave_bitonic_sort_u32(uint32_t (&k)[NPL], int lane) {
   constexpr int N = 64 * NPL;
 #pragma unroll
   for (int size = 2; size <= N; size <<= 1) {
@@ -229,14 +231,11 @@ __device__ __forceinline__ void wave_bitonic_sort(uint64_t (&k)[NPL], int lane) 
     for (int stride = size >> 1; stride > 0; stride >>= 1) {
       if (stride >= NPL) {
         const int lstride = stride / NPL;
-        const bool lower = (lane & lstride) == 0;
-        const bool up = (lane & (size / NPL)) == 0;
-        const bool keep_min = (lower == up);
+        const bool keep_min = ((lane & lstride) == 0) == ((lane & (size / NPL)) == 0);
 #pragma unroll
         for (int r = 0; r < NPL; ++r) {
-          const uint64_t o = shfl_xor_u64(k[r], lstride);
-          const bool take = keep_min ? (o < k[r]) : (o > k[r]);
-          k[r] = take ? o : k[r];
+          const uint32_t o = (uint32_t)__shfl_xor((int)k[r], lstride, 64);
+          k[r] = keep_min ? min(k[r], o) : max(k[r], o);
         }
       } else {
 #pragma unroll
@@ -244,10 +243,9 @@ __device__ __forceinline__ void wave_bitonic_sort(uint64_t (&k)[NPL], int lane) 
           if ((r & stride) == 0) {
             const int p = r | stride;
             const bool up = (size >= NPL) ? ((lane & (size / NPL)) == 0) : ((r & size) == 0);
-            const uint64_t x = k[r], y = k[p];
-            const bool sw = (x > y) == up;
-            k[r] = sw ? y : x;
-            k[p] = sw ? x : y;
+            const uint32_t lo = min(k[r], k[p]), hi = max(k[r], k[p]);
+            k[r] = up ? lo : hi;
+            k[p] = up ? hi : lo;
           }
         }
       }
@@ -344,11 +342,17 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
       }
     }
     if (!decided) {
-    wave_bitonic_sort<NPL>(k, lane);
+    // The sort runs on the 32-bit value keys alone (ascending key = descending value).  Entries of equal value are
+    // interchangeable in the running sum; which of them the stable order takes first matters only for the value at
+    // which the threshold is reached, and is settled there by index (below).
+    uint32_t kv[NPL], k0v[NPL];
+#pragma unroll
+    for (int r = 0; r < NPL; ++r) kv[r] = k0v[r] = (uint32_t)(k[r] >> 32);
+    wave_bitonic_sort_u32<NPL>(kv, lane);
 
     float v[NPL];
 #pragma unroll
-    for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < count) ? desc_key_value(k[r]) : 0.f;
+    for (int r = 0; r < NPL; ++r) v[r] = (lane * NPL + r < count) ? f32_from_orderable(~kv[r]) : 0.f;
     // parallel float64 prefix
     double loc[NPL];
     double c = 0.0;
@@ -402,9 +406,36 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
       }
     }
     if (first >= count) first = -1;   // never reached (padding ranks cannot qualify: they add zero)
+    if (first >= 0) {
+      // the selection is ranks 0 .. first of the stable order: every entry above the value at rank `first`, and of
+      // the entries equal to it the m lowest indices, m = first + 1 - (number of entries above it)
+      uint32_t mine = 0;
 #pragma unroll
-    for (int r = 0; r < NPL; ++r)
-      if (lane * NPL + r <= first) flag[(uint32_t)k[r]] = 1;
+      for (int r = 0; r < NPL; ++r) mine = (r == first % NPL) ? kv[r] : mine;
+      const uint32_t kstar = (uint32_t)__builtin_amdgcn_readlane((int)mine, first / NPL);
+      int above = 0, ties = 0;
+#pragma unroll
+      for (int r = 0; r < NPL; ++r) {
+        above += k0v[r] < kstar ? 1 : 0;
+        ties += k0v[r] == kstar ? 1 : 0;
+      }
+      int ties_incl = ties;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int t = __shfl_up(ties_incl, d, 64);
+        if (lane >= d) ties_incl += t;
+      }
+#pragma unroll
+      for (int off = 32; off > 0; off >>= 1) above += __shfl_xor(above, off, 64);
+      const int m = first + 1 - above;
+      int tie_rank = ties_incl - ties;   // ties at lower indices
+#pragma unroll
+      for (int r = 0; r < NPL; ++r) {
+        const bool tie = k0v[r] == kstar;
+        if (k0v[r] < kstar || (tie && tie_rank < m)) flag[lane * NPL + r] = 1;
+        tie_rank += tie ? 1 : 0;
+      }
+    }
     }   // !decided
     // a row without candidates is all zeros: sorted whole, its first entry is block 0 and the running sum is 0
     if (count == 0 && 0.0f >= thr && lane == 0) flag[0] = 1;
