@@ -132,6 +132,16 @@ int pbs_select_blocks(const float* block_attn_scores, const float* threshold_per
                       int32_t* csr_cols, int32_t* csr_cnt, uint8_t* block_needed, void* workspace,
                       size_t workspace_bytes, void* stream);
 
+/* Visit lists from a block mask somebody else made: csr_cols / csr_cnt as pbs_select_blocks writes them (the set
+ * key blocks of strictly earlier segments of every query block, ascending) from block_mask ((rows, nb, nb) bytes,
+ * non-zero = attend; entries of later segments are ignored: none of their keys is visible).  *own_missing (one int32
+ * the caller zeroes) receives the number of blocks of a query block's own segment the mask leaves out:
+ * pbs_sparse_attn_fwd always attends to the visible keys of the whole own segment, so a mask with own_missing != 0
+ * is not one it can serve.  For callers of the reference's attention stage that bring
+ * their own mask (pbs_attn/src/kernels/permuted_block_sparse_attention.py:134-157,314-323: block_mask argument). */
+int pbs_block_mask_to_csr(const uint8_t* block_mask, int32_t* csr_cols, int32_t* csr_cnt, int32_t* own_missing, int rows,
+                          int nb, int blocks_per_segment, void* stream);
+
 /* Block-sparse flash-attention forward.  Query block qb attends to the permuted K /
  * transposed V tiles listed in csr_cols (earlier segments, no element mask) and to
  * its own segment: blocks first-of-segment .. qb of the ORIGINAL k (B, Hkv, S, 128,

@@ -25,6 +25,7 @@ SIGNATURES = {
     "pbs_block_logits_softmax_causal": (c_int, [_P, _P, _P, _I, _I, _I, _P]),
     "pbs_select_blocks_workspace_bytes": (_Z, [_I]),
     "pbs_select_blocks": (c_int, [_P, _P, _F, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
+    "pbs_block_mask_to_csr": (c_int, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "pbs_sparse_attn_workspace_bytes": (c_size_t, [_I] * 4),
     "pbs_sparse_attn_fwd": (c_int, [_P] * 8 + [_I] * 7 + [_L] * 9 + [_F, _P, _P]),
     "pbs_sparse_attn_fwd_optional_diagonal": (c_int, [_P] * 9 + [_I] * 6 + [_L] * 9 + [_F, _P, _P]),

@@ -120,3 +120,59 @@ def permuted_block_selection(permuted_query_states: torch.Tensor, permuted_key_s
     kb = torch.arange(nb, device=dev).unsqueeze(0)
     segment_mask = (qb // bps) == (kb // bps)
     return scores, sel, segment_mask
+
+
+def sparse_attention_on_block_mask(perm_Q, perm_K, perm_V, perm_O, perm_Q_indices, perm_K_indices, perm_V_indices,
+                                   block_mask, block_size=128, segment_size=1024, causal=True):
+    """The reference's attention stage with its own argument list
+    (pbs_attn/src/kernels/permuted_block_sparse_attention.py:314-323, and the Triton launch of pbs.py:220-246):
+    queries in original order, K / V already permuted, their original positions, and a block mask in permuted
+    block coordinates.  Query i attends to permuted key j iff block_mask[block(i), block(j)] and
+    perm_K_indices[j] <= perm_Q_indices[i].  Fills and returns perm_O.
+
+    Runs on the HIP attention kernel, which reads a query block's own segment in original key order and always
+    attends to all of its visible keys: a mask that leaves out a block of a query block's own segment (the
+    reference's orchestrator never makes one, pbs.py:209) raises ValueError, as do permuted queries."""
+    assert causal
+    assert segment_size % block_size == 0, "segment_size must be a multiple of block_size"
+    B, H, S, D = perm_Q.shape
+    assert perm_K.shape[2] == S, "Only support prefilling for now"
+    dev = perm_Q.device
+    nb = (S + block_size - 1) // block_size
+    pos = torch.arange(S, device=dev)
+    if not bool((perm_Q_indices.to(dev) == pos.view(1, 1, -1)).all()):
+        raise ValueError("the HIP attention kernel takes queries in their original order (the reference never permutes them)")
+    if block_mask.shape[-2:] != (nb, nb):
+        raise ValueError(f"block_mask must be (..., {nb}, {nb}) for {S} tokens in blocks of {block_size}")
+    k, v = perm_K, perm_V
+    if k.shape[1] != H:
+        k = k.repeat_interleave(H // k.shape[1], dim=1)
+        v = v.repeat_interleave(H // v.shape[1], dim=1)
+    k_idx = perm_K_indices.to(device=dev, dtype=torch.int32).expand(B, H, -1).contiguous()
+    v_idx = perm_V_indices.to(device=dev, dtype=torch.int32).expand(B, H, -1).contiguous()
+    # back to original key order (the scatter kernel of the output un-permutation), then the kernels' own layouts
+    k_orig = ops.unpermute(k.contiguous(), k_idx, torch.empty_like(k, memory_format=torch.contiguous_format))
+    v_orig = ops.unpermute(v.contiguous(), v_idx, torch.empty_like(v, memory_format=torch.contiguous_format))
+    pad_idx = torch.cat([k_idx, torch.arange(S, nb * block_size, dtype=torch.int32, device=dev).expand(B, H, -1)], dim=-1)
+    perm_k, perm_vt, _, orig_vt = ops.gather_kv(k_orig, v_orig, pad_idx.contiguous(), H, want_orig_vt=True, want_pooled=False)
+    cols, cnt, missing = ops.block_mask_to_csr(block_mask.to(dev).expand(B, H, nb, nb), segment_size // block_size)
+    if int(missing.item()) != 0:
+        raise ValueError("block_mask leaves out blocks of a query block's own segment: the HIP attention kernel "
+                         "always attends to the visible keys of the whole own segment (as pbs.py:209 arranges)")
+    out = ops.sparse_attn_fwd(perm_Q, perm_k, perm_vt, k_orig, orig_vt, cols, cnt, segment_size, 1.0 / (D ** 0.5))
+    perm_O.copy_(out)
+    return perm_O
+
+
+class _TritonStyleLauncher:
+    """``kernel[grid](...)`` with the positional list of the reference's Triton kernel
+    (pbs_attn/src/pbs.py:220-246): the tensors and the two size constants are used, strides come from the tensors."""
+
+    def __getitem__(self, grid):
+        def launch(Q, K, V, O, block_mask, q_idx, k_idx, v_idx, *strides_and_sizes, LOGICAL_BLOCK_SIZE=128,
+                   SEGMENT_SIZE=1024, **meta):
+            sparse_attention_on_block_mask(Q, K, V, O, q_idx, k_idx, v_idx, block_mask, LOGICAL_BLOCK_SIZE, SEGMENT_SIZE, True)
+        return launch
+
+
+permuted_block_sparse_attn_kernel = _TritonStyleLauncher()

@@ -468,7 +468,46 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
   if (lane == 0) a.csr_cnt[(int64_t)row * nb + qb] = base;
 }
 
+// Visit lists from a given block mask: one wave per (row, query block), the set bits of strictly earlier segments
+// compacted in ascending order; own_missing counts the blocks of the query block's own segment the mask leaves out
+// (in permuted order any of them can hold keys the query may see).
+__global__ __launch_bounds__(256) void mask_to_csr_kernel(const uint8_t* __restrict__ mask, int32_t* __restrict__ cols,
+                                                          int32_t* __restrict__ cnt, int32_t* __restrict__ own_missing, int nb,
+                                                          int bps, int total_rows) {
+  const int lane = threadIdx.x & 63;
+  const int64_t rq = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (rq >= total_rows) return;
+  const int qb = (int)(rq % nb);
+  const int seg_first = (qb / bps) * bps, seg_end = min(seg_first + bps, nb);
+  const uint8_t* m = mask + rq * nb;
+  int base = 0, missing = 0;
+  for (int kb0 = 0; kb0 < seg_end; kb0 += 64) {
+    const int kb = kb0 + lane;
+    const bool on = kb < seg_end && m[kb] != 0;
+    const bool visit = on && kb < seg_first;
+    const uint64_t ballot = __ballot(visit);
+    if (visit) cols[rq * nb + base + __popcll(ballot & ((1ull << lane) - 1ull))] = kb;
+    base += __popcll(ballot);
+    missing += __popcll(__ballot(kb >= seg_first && kb < seg_end && !on));
+  }
+  if (lane == 0) {
+    cnt[rq] = base;
+    if (missing) atomicAdd(own_missing, missing);
+  }
+}
+
 }  // namespace
+
+extern "C" int pbs_block_mask_to_csr(const uint8_t* block_mask, int32_t* csr_cols, int32_t* csr_cnt, int32_t* own_missing,
+                                     int rows, int nb, int blocks_per_segment, void* stream) {
+  PBS_REQUIRE(block_mask && csr_cols && csr_cnt && own_missing, "pbs_block_mask_to_csr: null pointer");
+  PBS_REQUIRE(rows > 0 && nb > 0 && nb <= 4096 && blocks_per_segment > 0 && (int64_t)rows * nb < (1ll << 31),
+              "pbs_block_mask_to_csr: bad shape");
+  const int total = rows * nb;
+  hipLaunchKernelGGL(mask_to_csr_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, (hipStream_t)stream, block_mask,
+                     csr_cols, csr_cnt, own_missing, nb, blocks_per_segment, total);
+  return pbs_check_launch("pbs_block_mask_to_csr");
+}
 
 extern "C" size_t pbs_select_blocks_workspace_bytes(int rows) { return (size_t)rows * sizeof(int32_t); }
 

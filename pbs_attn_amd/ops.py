@@ -224,6 +224,24 @@ def select_blocks(block_attn_scores, threshold, idx, seq_len, block_size, segmen
     return sel, fin, cols, cnt
 
 
+def block_mask_to_csr(block_mask, blocks_per_segment):
+    """Visit lists (csr_cols, csr_cnt) of a (B, H, nb, nb) bool block mask made elsewhere, and the number of
+    own-segment blocks it leaves out (a device tensor of one int32; the attention kernel always attends to the
+    visible keys of the whole own segment)."""
+    lib = _lib.load()
+    if not block_mask.is_cuda:
+        raise _lib.PbsHipError("PBS HIP kernels need tensors on the GPU (there is no CPU path)")
+    B, H, nb, nb2 = block_mask.shape
+    assert nb == nb2, "only square (prefill) block masks are supported"
+    m = block_mask.to(torch.uint8).contiguous()
+    cols = torch.empty((B, H, nb, nb), dtype=torch.int32, device=m.device)
+    cnt = torch.empty((B, H, nb), dtype=torch.int32, device=m.device)
+    missing = torch.zeros(1, dtype=torch.int32, device=m.device)
+    _lib.check(lib.pbs_block_mask_to_csr(_ptr(m), _ptr(cols), _ptr(cnt), _ptr(missing), B * H, nb, blocks_per_segment,
+                                         _stream()), "pbs_block_mask_to_csr")
+    return cols, cnt, missing
+
+
 def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None,
                     own_block_needed=None):
     """Attention of every query block over the permuted tiles listed in the CSR (earlier segments) and

@@ -105,6 +105,10 @@ def test_reference_callers_import_lines_work():
     from pbs_attn.src.pbs import first_token_mask, permuted_block_selection
     from pbs_attn.src.pbs import apply_permutation as ap2
     from pbs_attn.baselines.MeanPooling import MeanPooling_prefill
+    # pbs_attn/src/pbs.py:6 of the reference
+    from pbs_attn.src.kernels.permuted_block_sparse_attention import (  # noqa: F401
+        _permuted_block_sparse_attn_fwd, _permuted_block_sparse_attn_fwd_torch_naive)
+    assert callable(_permuted_block_sparse_attn_fwd_torch_naive) and callable(_permuted_block_sparse_attn_fwd[(1, 1, 1)])
     assert ap2 is apply_permutation
 
     def params(fn):

@@ -157,3 +157,45 @@ def test_query_blocks_that_select_nothing_give_zeros(dev, B, Hq, Hkv, S, thr):
         own_mask = got["block_mask"].cpu()
         dense2 = torch.nan_to_num(O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], own_mask, 128), nan=0.0)
         assert_attn_close(out2.cpu(), dense2, what="MeanPooling_prefill with unreachable threshold vs dense fp32 on its own mask")
+
+
+def test_attention_stage_with_the_reference_argument_list(dev):
+    """pbs_attn.src.kernels.permuted_block_sparse_attention: the attention stage under the reference's two names
+    (the naive function's argument list, kernels/...:314-323, and the Triton kernel's launch form, pbs.py:220-246), fed
+    with what the reference's orchestrator hands it: permuted K / V, their original positions, block_mask | segment_mask."""
+    from pbs_attn.src.kernels.permuted_block_sparse_attention import (
+        _permuted_block_sparse_attn_fwd, _permuted_block_sparse_attn_fwd_torch_naive)
+    B, H, S, seg, thr = 2, 3, 1664, 512, 0.7
+    q, k, v = small_case(B, H, H, S, seed=29)
+    ref_out, mid = O.permuted_block_sparse_attn_fwd(q, k, v, 128, seg, thr, return_intermediates=True)
+    idx, mask = mid["key_indices"], mid["final_mask"]
+    perm_k, perm_v = O.gather_rows(k, idx), O.gather_rows(v, idx)
+    dense = O.dense_masked_attention_fp32(q, perm_k, perm_v, idx, mask, 128)
+    q_idx = torch.arange(S).view(1, 1, -1).expand(B, H, -1)
+    args = [t.to(dev) for t in (q, perm_k, perm_v)]
+    out = torch.empty_like(args[0])
+    got = _permuted_block_sparse_attn_fwd_torch_naive(*args, out, q_idx.to(dev), idx.to(dev), idx.to(dev), mask.to(dev), 128, seg, True)
+    assert got is out
+    assert_attn_close(out.cpu(), dense, what="attention stage on the oracle's mask vs dense fp32")
+    assert_attn_close(out.cpu(), ref_out, max_abs=2.5e-2, what="attention stage vs the oracle's naive path")
+    out2 = torch.zeros_like(out)
+    strides = [0] * 29
+    _permuted_block_sparse_attn_fwd[(13, H, B)](*args, out2, mask.to(dev), q_idx.to(dev), idx.to(dev), idx.to(dev), *strides, S, S,
+                                               128 ** -0.5, H=H, num_kv_groups=1, HEAD_DIM=128, SEGMENT_SIZE=seg,
+                                               LOGICAL_BLOCK_SIZE=128, STAGE=3)
+    assert torch.equal(out2, out)
+    # the visit lists made from the mask are the selection's own
+    cols, cnt, missing = ops.block_mask_to_csr(mask.to(dev), seg // 128)
+    nb, bps = mask.shape[-1], seg // 128
+    qb = torch.arange(nb)
+    earlier = (qb.view(1, -1) // bps) < (qb.view(-1, 1) // bps)
+    assert int(missing.item()) == 0 and torch.equal(cnt.cpu(), (mask & earlier).sum(-1).int())
+    row = cols[1, 2, nb - 1, :cnt[1, 2, nb - 1]].cpu()
+    assert torch.equal(row, torch.where(mask[1, 2, nb - 1] & earlier[nb - 1])[0].int())
+    # a mask without a block of the own segment, and permuted queries, are refused
+    bad = mask.clone()
+    bad[0, 0, 5, 5] = False
+    with pytest.raises(ValueError, match="own segment"):
+        _permuted_block_sparse_attn_fwd_torch_naive(*args, out, q_idx.to(dev), idx.to(dev), idx.to(dev), bad.to(dev), 128, seg, True)
+    with pytest.raises(ValueError, match="original order"):
+        _permuted_block_sparse_attn_fwd_torch_naive(*args, out, q_idx.flip(-1).to(dev), idx.to(dev), idx.to(dev), mask.to(dev), 128, seg, True)
