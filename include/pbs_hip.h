@@ -104,6 +104,13 @@ int pbs_pool_q(const void* q, void* pooled_q, int B, int Hq, int S, int head_dim
 int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows, int nb,
                              int head_dim, int blocks_per_segment, void* stream);
 
+/* pbs_block_logits_softmax for a consumer that reads a row's candidate entries only (pbs_select_blocks with
+ * candidate_rule 1 on at most 1024 blocks): the zeros outside the candidates and the NaN rows are not written, which
+ * halves the kernel's stores.  The candidate entries are the bits pbs_block_logits_softmax writes.  Replaces the
+ * same lines, pbs_attn/src/pbs.py:97-107 and pbs_attn/src/utils.py:30-33. */
+int pbs_block_logits_softmax_candidates_only(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows,
+                                             int nb, int head_dim, int blocks_per_segment, void* stream);
+
 /* The same with the candidate rule of the reference's un-permuted MeanPooling baseline: query block qb
  * scores every key block kb <= qb (the causal lower triangle INCLUDING the diagonal), so no row is NaN.
  * Replaces pbs_attn/baselines/MeanPooling.py:43-48 (mask) + pbs_attn/src/utils.py:30-33. */

@@ -22,6 +22,7 @@ SIGNATURES = {
     "pbs_pool_blocks": (c_int, [_P] * 6 + [_I] * 6 + [_L] * 6 + [_I, _I, _P]),
     "pbs_pool_q": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P]),
     "pbs_block_logits_softmax": (c_int, [_P, _P, _P, _I, _I, _I, _I, _P]),
+    "pbs_block_logits_softmax_candidates_only": (c_int, [_P, _P, _P, _I, _I, _I, _I, _P]),
     "pbs_block_logits_softmax_causal": (c_int, [_P, _P, _P, _I, _I, _I, _P]),
     "pbs_select_blocks_workspace_bytes": (_Z, [_I]),
     "pbs_select_blocks": (c_int, [_P, _P, _F, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),

@@ -29,7 +29,9 @@ __device__ __forceinline__ int candidate_count(int qb, int bps) {
   return CAUSAL ? qb + 1 : (qb / bps) * bps;
 }
 
-template <bool CAUSAL>
+// CANDIDATES_ONLY: only the candidate entries of a row are written (the selection that follows on the single-call path
+// reads no others); otherwise all nb columns, zeros outside the candidates and NaN rows where there are none.
+template <bool CAUSAL, bool CANDIDATES_ONLY>
 __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_t* pooled_q, const uint16_t* pooled_k,
                                                                    float* P, int nb, int bps, float sqrt_d) {
   __shared__ float s_m[4][32], s_l[4][32];
@@ -103,7 +105,7 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
   bf16x8 qa[8];
 #pragma unroll
   for (int t = 0; t < 8; ++t) qa[t] = qf[t];
-  for (int kt = wave; kt < n_kt_all; kt += 4) {
+  for (int kt = wave; kt < (CANDIDATES_ONLY ? n_kt_cand : n_kt_all); kt += 4) {
     const int kb = 32 * kt + j;
     f32x16 acc = {0};
     if (kt < n_kt_cand) {
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
         if (cand == 0) p = __uint_as_float(0x7fc00000u);
         else if (kb < cand) p = __expf(logit_round(acc[r], sqrt_d) - s_max[ql]) * s_inv[ql];
         else p = 0.f;
-        out[(int64_t)qb * nb + kb] = p;
+        if (!CANDIDATES_ONLY || kb < cand) out[(int64_t)qb * nb + kb] = p;
       }
     }
   }
@@ -130,18 +132,21 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
 }  // namespace
 
 namespace {
-int launch_block_logits(const char* who, bool causal, const void* pooled_q, const void* pooled_k, float* block_attn_scores,
+int launch_block_logits(const char* who, bool causal, bool candidates_only, const void* pooled_q, const void* pooled_k, float* block_attn_scores,
                         int rows, int nb, int head_dim, int blocks_per_segment, void* stream) {
   PBS_REQUIRE(pooled_q && pooled_k && block_attn_scores, "%s: null tensor pointer", who);
   PBS_REQUIRE(head_dim == D, "%s: head_dim must be 128, got %d", who, head_dim);
   PBS_REQUIRE(rows > 0 && rows <= 65535 && nb > 0 && blocks_per_segment > 0, "%s: bad shape", who);
   const dim3 grid((nb + 31) / 32, rows);
   const float sqrt_d = (float)sqrt((double)head_dim);
-  if (causal)
-    hipLaunchKernelGGL(block_logits_softmax_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
+  if (candidates_only)
+    hipLaunchKernelGGL((block_logits_softmax_kernel<false, true>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
+                       (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);
+  else if (causal)
+    hipLaunchKernelGGL((block_logits_softmax_kernel<true, false>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
                        (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);
   else
-    hipLaunchKernelGGL(block_logits_softmax_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
+    hipLaunchKernelGGL((block_logits_softmax_kernel<false, false>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
                        (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);
   return pbs_check_launch(who);
 }
@@ -149,12 +154,18 @@ int launch_block_logits(const char* who, bool causal, const void* pooled_q, cons
 
 extern "C" int pbs_block_logits_softmax(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows,
                                         int nb, int head_dim, int blocks_per_segment, void* stream) {
-  return launch_block_logits("pbs_block_logits_softmax", false, pooled_q, pooled_k, block_attn_scores, rows, nb, head_dim,
+  return launch_block_logits("pbs_block_logits_softmax", false, false, pooled_q, pooled_k, block_attn_scores, rows, nb, head_dim,
                              blocks_per_segment, stream);
 }
 
 extern "C" int pbs_block_logits_softmax_causal(const void* pooled_q, const void* pooled_k, float* block_attn_scores,
                                                int rows, int nb, int head_dim, void* stream) {
-  return launch_block_logits("pbs_block_logits_softmax_causal", true, pooled_q, pooled_k, block_attn_scores, rows, nb,
+  return launch_block_logits("pbs_block_logits_softmax_causal", true, false, pooled_q, pooled_k, block_attn_scores, rows, nb,
                              head_dim, 1, stream);
+}
+
+extern "C" int pbs_block_logits_softmax_candidates_only(const void* pooled_q, const void* pooled_k, float* block_attn_scores, int rows,
+                                             int nb, int head_dim, int blocks_per_segment, void* stream) {
+  return launch_block_logits("pbs_block_logits_softmax", false, true, pooled_q, pooled_k, block_attn_scores, rows, nb, head_dim,
+                             blocks_per_segment, stream);
 }

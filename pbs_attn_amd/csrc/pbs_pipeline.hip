@@ -115,8 +115,14 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
     if ((rc = pbs_pool_blocks(q, k, (const int32_t*)(w + L.idx), w + L.pooled_q, w + L.pooled_k, needed, B, Hq, Hkv, S,
                               head_dim, block_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, query_pool_max, key_pool_max,
                               stream))) return rc;
-    if ((rc = pbs_block_logits_softmax(w + L.pooled_q, w + L.pooled_k, (float*)(w + L.probs), rows, nb, head_dim,
-                                       segment_size / block_size, stream))) return rc;
+    // (up to 1024 blocks the selection reads a row's candidate entries only: the others are not written)
+    if (nb <= 1024) {
+      if ((rc = pbs_block_logits_softmax_candidates_only(w + L.pooled_q, w + L.pooled_k, (float*)(w + L.probs), rows, nb,
+                                                         head_dim, segment_size / block_size, stream))) return rc;
+    } else {
+      if ((rc = pbs_block_logits_softmax(w + L.pooled_q, w + L.pooled_k, (float*)(w + L.probs), rows, nb, head_dim,
+                                         segment_size / block_size, stream))) return rc;
+    }
   }
   if ((rc = pbs_select_blocks((const float*)(w + L.probs), threshold_per_row, threshold, threshold_is_int_one,
                               force_select_first_block, /*candidate_rule=*/1, (const int32_t*)(w + L.idx), rows, S, block_size,

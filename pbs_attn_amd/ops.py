@@ -175,16 +175,23 @@ def pool_q(q, query_pool_mode="mean"):
     return pooled
 
 
-def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment, causal_candidates=False):
+def block_logits_softmax(pooled_q, pooled_k, blocks_per_segment, causal_candidates=False, candidates_only=False):
     """(B, H, nb, nb) float32 block probabilities; utils.py:30-33.  Candidates of a query block are the key
     blocks of strictly earlier segments (pbs.py:97-107) or, with ``causal_candidates``, every block up to and
-    including the diagonal one (baselines/MeanPooling.py:43-48)."""
+    including the diagonal one (baselines/MeanPooling.py:43-48).  ``candidates_only`` (earlier-segment rule): the
+    entries outside a row's candidates stay unwritten -- for ``select_blocks(..., candidate_rule=1)`` on at most 1024
+    blocks, which reads no others."""
     _check_bf16_cuda(pooled_q, pooled_k)
     lib = _lib.load()
     pooled_q, pooled_k = pooled_q.contiguous(), pooled_k.contiguous()
     B, H, nb, D = pooled_q.shape
     P = torch.empty((B, H, nb, nb), dtype=torch.float32, device=pooled_q.device)
-    if causal_candidates:
+    if candidates_only:
+        assert not causal_candidates
+        _lib.check(lib.pbs_block_logits_softmax_candidates_only(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D,
+                                                                blocks_per_segment, _stream()),
+                   "pbs_block_logits_softmax_candidates_only")
+    elif causal_candidates:
         _lib.check(lib.pbs_block_logits_softmax_causal(_ptr(pooled_q), _ptr(pooled_k), _ptr(P), B * H, nb, D, _stream()),
                    "pbs_block_logits_softmax_causal")
     else:

@@ -119,7 +119,7 @@ def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment
 
 
 def _select_then_gather(query_states, key_states, value_states, block_size, segment_size, threshold,
-                        force_select_first_block, query_pool_mode, key_pool_mode):
+                        force_select_first_block, query_pool_mode, key_pool_mode, candidates_only=False):
     B, Hq, S, _ = query_states.shape
     s_pad = (S + block_size - 1) // block_size * block_size
     nseg, rem = S // segment_size, S % segment_size
@@ -132,7 +132,9 @@ def _select_then_gather(query_states, key_states, value_states, block_size, segm
         _mark("sort")
     pooled_q, pooled_k, needed = ops.pool_blocks(query_states, key_states, idx, query_pool_mode, key_pool_mode)
     _mark("pool")
-    P = ops.block_logits_softmax(pooled_q, pooled_k, segment_size // block_size)
+    # candidates_only (the single-call path's form, up to 1024 blocks): the selection reads a row's candidate entries only
+    P = ops.block_logits_softmax(pooled_q, pooled_k, segment_size // block_size,
+                                 candidates_only=candidates_only and s_pad // block_size <= 1024)
     _mark("estimate")
     _, _, cols, cnt = ops.select_blocks(P, threshold, idx, S, block_size, segment_size, force_select_first_block,
                                         want_masks=False, block_needed=needed, candidate_rule=1)
@@ -197,7 +199,7 @@ def permuted_block_sparse_attn_fwd(
         # the order of the single-call path: the estimate runs on key blocks pooled straight from K, and K / V
         # are gathered after the selection, only the blocks some query block visits
         perm, sel = _select_then_gather(query_states, key_states, value_states, block_size, segment_size, threshold,
-                                        force_select_first_block, query_pool_mode, key_pool_mode)
+                                        force_select_first_block, query_pool_mode, key_pool_mode, candidates_only=True)
     out = perm.attention(query_states, sel["csr_cols"], sel["csr_cnt"], segment_size, 1.0 / math.sqrt(head_dim))
     _mark("sparse_attn")
     # queries are not permuted (pbs.py:191-193): un-permutation is the identity
