@@ -95,7 +95,7 @@ def load_probe_library():
         from pbs_attn_amd import _lib
         _lib.load()   # the probe library takes its error helpers from the operator's library
         lib = ctypes.CDLL(os.path.join(os.path.dirname(_lib.LIB_PATH), "libpbs_probe.so"))
-        lib.pbs_mfma_probe.restype, lib.pbs_mfma_probe.argtypes = c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p]
+        lib.pbs_mfma_probe.restype, lib.pbs_mfma_probe.argtypes = c_int, [c_void_p, c_int, c_int, c_void_p, c_void_p, c_void_p]
         lib.pbs_mfma_probe_flop.restype, lib.pbs_mfma_probe_flop.argtypes = c_double, [c_int]
         lib.pbs_attn_tile_probe.restype = c_int
         lib.pbs_attn_tile_probe.argtypes = [c_void_p, c_int, c_int, c_int, c_void_p, c_void_p, c_void_p]
@@ -103,10 +103,11 @@ def load_probe_library():
     return _probe_lib
 
 
-def mfma_ceiling(torch, iters=200000):
-    """What a loop of nothing but bf16 MFMAs sustains on this GPU right now, on all-zero operands and on
-    normally distributed ones (the rate depends on the values: the chip lowers its clock to stay inside its
-    power limit).  The second figure is the practical ceiling for a kernel fed with data like attention's."""
+def mfma_ceiling(torch, iters=100000):
+    """What the matrix cores sustain on this GPU by themselves, on all-zero operands and on normally distributed
+    ones (the rate depends on the values: the chip lowers its clock to stay inside its power limit), with the
+    attention kernel's instruction (v_mfma_f32_16x16x32_bf16) and, for comparison, with v_mfma_f32_32x32x16_bf16.
+    `normal` is the practical ceiling for a kernel fed with data like attention's."""
     from pbs_attn_amd import _lib
     lib = load_probe_library()
     dev = torch.device("cuda")
@@ -115,21 +116,23 @@ def mfma_ceiling(torch, iters=200000):
     pools = {"zeros": torch.zeros(65536, dtype=torch.bfloat16, device=dev),
              "normal": torch.randn(65536, generator=gen).to(torch.bfloat16).to(dev)}
     st = torch.cuda.current_stream().cuda_stream
-    out = {"unit": "TFLOP/s", "kernel": "v_mfma_f32_32x32x16_bf16 only, 256 workgroups x 8 waves"}
-    for name, pool in pools.items():
-        clocks = torch.zeros(2, dtype=torch.int64, device=dev)
-        _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), 2000, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
-        torch.cuda.synchronize()
-        clocks.zero_()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), iters, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
-        e1.record()
-        torch.cuda.synchronize()
-        ms = e0.elapsed_time(e1)
-        c = clocks.tolist()
-        out[name] = lib.pbs_mfma_probe_flop(iters) / ms / 1e9
-        out[name + "_shader_clock_mhz"] = 100.0 * c[0] / max(1, c[1])
+    out = {"unit": "TFLOP/s", "kernel": "matrix instructions only, 256 workgroups x 8 waves: v_mfma_f32_16x16x32_bf16 "
+                                        "(the attention kernel's; keys `zeros`, `normal`) and v_mfma_f32_32x32x16_bf16 (`*_32x32x16`)"}
+    for shape, suffix in ((0, ""), (1, "_32x32x16")):
+        for name, pool in pools.items():
+            clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+            _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), 2000, shape, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
+            torch.cuda.synchronize()
+            clocks.zero_()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            _lib.check(lib.pbs_mfma_probe(pool.data_ptr(), iters, shape, sink.data_ptr(), clocks.data_ptr(), st), "pbs_mfma_probe")
+            e1.record()
+            torch.cuda.synchronize()
+            ms = e0.elapsed_time(e1)
+            c = clocks.tolist()
+            out[name + suffix] = lib.pbs_mfma_probe_flop(iters) / ms / 1e9
+            out[name + suffix + "_shader_clock_mhz"] = 100.0 * c[0] / max(1, c[1])
     return out
 
 

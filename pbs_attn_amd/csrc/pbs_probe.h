@@ -5,12 +5,13 @@
 extern "C" {
 #endif
 
-/* `iters` x 8 v_mfma_f32_32x32x16_bf16 per wave on
+/* A loop of matrix instructions only: per wave `iters` x 16 v_mfma_f32_16x16x32_bf16 (the attention kernel's) or,
+ * shape_32x32x16 != 0, `iters` x 8 v_mfma_f32_32x32x16_bf16 (the same FLOP), on
  * 256 workgroups of 8 waves, operands taken from `operands` (65536 bf16 values of the caller's choice: the
  * sustained rate depends on the values).  `sink` takes 256 * 512 floats, `clocks` (two 64-bit counters the
  * caller zeroes) accumulates shader-clock and 100 MHz ticks over the workgroups; time the launch with
  * events.  pbs_mfma_probe_flop gives the FLOP count of one launch. */
-int pbs_mfma_probe(const void* operands, int iters, float* sink, unsigned long long* clocks, void* stream);
+int pbs_mfma_probe(const void* operands, int iters, int shape_32x32x16, float* sink, unsigned long long* clocks, void* stream);
 double pbs_mfma_probe_flop(int iters);
 
 /* the attention kernel's tile pipeline alone.  256

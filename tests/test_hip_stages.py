@@ -468,8 +468,9 @@ def test_mfma_probe_runs_and_counts_clocks(dev):
     pool = torch.randn(65536, device=dev).bfloat16()
     sink = torch.empty(256 * 512, dtype=torch.float32, device=dev)
     clocks = torch.zeros(2, dtype=torch.int64, device=dev)
-    rc = lib.pbs_mfma_probe(pool.data_ptr(), 100, sink.data_ptr(), clocks.data_ptr(), torch.cuda.current_stream().cuda_stream)
-    assert rc == 0
+    for shape in (0, 1):
+        rc = lib.pbs_mfma_probe(pool.data_ptr(), 100, shape, sink.data_ptr(), clocks.data_ptr(), torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
     torch.cuda.synchronize()
     c = clocks.tolist()
     assert c[0] > 0 and c[1] > 0 and torch.isfinite(sink).all()
