@@ -310,11 +310,8 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
     score_b = kv_once + B * Hq * bs * D * e + B * Hq * S * 4
     pool_b = kv_once + B * Hq * S * 4 + 2 * B * Hq * nb * D * e + B * Hq * S * D * e    # K, indices, Q in; pooled out
     # reads: the K and V rows of the gathered blocks (each row counted once per KV head at most) and their indices;
-    # writes: the gathered tiles.  The original-order transposed copy of V that the same launch writes for the
-    # attention kernel's own-segment tiles (V read once more, the copy written) is this design's own extra traffic
-    # and is reported beside the rate, not in it.
+    # writes: the gathered tiles.
     gather_b = 2 * min(f * B * Hq, B * Hkv) * S * D * e + f * B * Hq * S * 4 + 2 * f * B * Hq * S * D * e
-    res["gather_extra_bytes_orig_vt"] = 2 * kv_once
     est_b = (0 if "pool" in stages else B * Hq * S * D * e) + 2 * B * Hq * nb * D * e + B * Hq * nb * nb * 4
     res["hbm_gbs"] = {
         "score": score_b / (stages["score"] * 1e-3) / 1e9 if "score" in stages else None,
@@ -327,7 +324,7 @@ def run_workload(torch, name, steps, warmup, seed=0, overrides=None, with_dense=
         # delivers when the matrix cores draw the least power
         from pbs_attn_amd import ops
         zq, zk, zv = torch.zeros_like(q), torch.zeros_like(perm.perm_k), torch.zeros_like(perm.perm_vt)
-        zargs = (zq, zk, zv, torch.zeros_like(k), torch.zeros_like(perm.orig_vt), sel["csr_cols"], sel["csr_cnt"], seg)
+        zargs = (zq, zk, zv, torch.zeros_like(k), torch.zeros_like(v), sel["csr_cols"], sel["csr_cnt"], seg)
         ops.sparse_attn_fwd(*zargs)
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
@@ -544,7 +541,6 @@ def main():
         "ms_per_step_staged": res["ms_per_step_staged"],
         "hbm_gbs": res["hbm_gbs"],
         "gathered_block_fraction": res["gathered_block_fraction"],
-        "gather_extra_bytes_orig_vt": res["gather_extra_bytes_orig_vt"],
         "dense_sdpa_ms": res.get("dense_sdpa_ms"),
         "dense_own_kernel_ms": res.get("dense_own_kernel_ms"),
         "speedup_vs_dense_sdpa": res.get("speedup_vs_dense_sdpa"),

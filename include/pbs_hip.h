@@ -61,17 +61,13 @@ int pbs_segment_argsort(const float* scores, int32_t* key_indices, int rows, int
 
 /* Gather K and V into permuted order and pool the permuted key blocks.
  * perm_k: (B, Hq, nb*128, 128) rows past S zero; perm_vt: (B, Hq, nb, 128, 128)
- * holding each V block transposed [d][key]; pooled_k: (B, Hq, nb, 128) bf16;
- * orig_vt (may be null): (B, Hkv, nb, 128, 128), the V blocks in ORIGINAL key order,
- * transposed the same way and zero past S -- the attention kernel reads a query
- * block's own segment un-permuted, where the causal mask is a plain triangle.
- * pooled_k may be null (no pooling).  block_needed (may be null): (B*Hq, nb) bytes as written by
+ * holding each V block transposed [d][key]; pooled_k: (B, Hq, nb, 128) bf16, may be null (no pooling).  block_needed (may be null): (B*Hq, nb) bytes as written by
  * pbs_select_blocks; permuted blocks whose byte is zero are skipped and their perm_k / perm_vt
  * tiles left unwritten (the attention kernel reads only the blocks on some visit list).
  * Replaces pbs_attn/src/permute_states.py:59-69, pbs_attn/src/pbs.py:213-215,
  * the key padding of pbs.py:78-79 and the key pooling of pbs_attn/src/utils.py:24-29. */
 int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
-                  void* pooled_k, void* orig_vt, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
+                  void* pooled_k, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
                   int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
                   const uint8_t* block_needed, void* stream);
 
@@ -151,8 +147,8 @@ int pbs_block_mask_to_csr(const uint8_t* block_mask, int32_t* csr_cols, int32_t*
 
 /* Block-sparse flash-attention forward.  Query block qb attends to the permuted K /
  * transposed V tiles listed in csr_cols (earlier segments, no element mask) and to
- * its own segment: blocks first-of-segment .. qb of the ORIGINAL k (B, Hkv, S, 128,
- * caller's strides) and orig_vt, with the causal triangle on block qb.  The keys a
+ * its own segment: blocks first-of-segment .. qb of the ORIGINAL k and v (B, Hkv, S, 128,
+ * caller's strides, read in place), with the causal triangle on block qb.  The keys a
  * query sees are exactly those of the reference's final mask and element mask
  * (a segment's permuted blocks hold the same keys as its original blocks).
  * out: (B, Hq, S, 128) bf16 with its own strides, original query order.
@@ -162,11 +158,11 @@ int pbs_block_mask_to_csr(const uint8_t* block_mask, int32_t* csr_cols, int32_t*
  * Replaces pbs_attn/src/kernels/permuted_block_sparse_attention.py:134-311
  * (launch at pbs_attn/src/pbs.py:220-246). */
 size_t pbs_sparse_attn_workspace_bytes(int B, int Hq, int S, int segment_size);
-int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* v,
                         const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
                         int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                        int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                        float softmax_scale, void* workspace, void* stream);
+                        int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                        int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale, void* workspace, void* stream);
 
 /* pbs_sparse_attn_fwd for one-block segments (segment_size = block_size: the un-permuted MeanPooling mode) with an
  * OPTIONAL diagonal block: query block qb of head row r attends to its own block (with the causal triangle) only
@@ -176,11 +172,12 @@ int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, 
  * block_size).  Replaces the attention call of pbs_attn/baselines/MeanPooling.py:80-96 when
  * force_select_current_block (:54-58) is off. */
 int pbs_sparse_attn_fwd_optional_diagonal(const void* q, const void* perm_k, const void* perm_vt, const void* k,
-                                          const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt,
+                                          const void* v, const int32_t* csr_cols, const int32_t* csr_cnt,
                                           const uint8_t* own_block_needed, void* out, int B, int Hq, int Hkv, int S,
                                           int head_dim, int block_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                                          int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh,
-                                          int64_t o_ss, float softmax_scale, void* workspace, void* stream);
+                                          int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh,
+                                          int64_t v_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale,
+                                          void* workspace, void* stream);
 
 /* out[b,h,q_idx[b,h,i],:] = o_perm[b,h,i,:] (o_perm contiguous).  q_idx null with
  * o_perm == out is the identity fast path (no launch): the reference does not

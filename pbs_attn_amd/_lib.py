@@ -17,7 +17,7 @@ SIGNATURES = {
     "pbs_score_keys": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P, _Z, _P]),
     "pbs_score_keys_static": (c_int, [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _L, _L, _L, _L, _L, _L, _P]),
     "pbs_segment_argsort": (c_int, [_P, _P, _I, _I, _I, _I, _P]),
-    "pbs_gather_kv": (c_int, [_P] * 7 + [_I] * 6 + [_L] * 6 + [_I, _P, _P]),
+    "pbs_gather_kv": (c_int, [_P] * 6 + [_I] * 6 + [_L] * 6 + [_I, _P, _P]),
     "pbs_pool_k_permuted": (c_int, [_P] * 4 + [_I] * 6 + [_L] * 3 + [_I, _P]),
     "pbs_pool_blocks": (c_int, [_P] * 6 + [_I] * 6 + [_L] * 6 + [_I, _I, _P]),
     "pbs_pool_q": (c_int, [_P, _P, _I, _I, _I, _I, _I, _L, _L, _L, _I, _P]),
@@ -28,8 +28,8 @@ SIGNATURES = {
     "pbs_select_blocks": (c_int, [_P, _P, _F, _I, _I, _I, _P, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _Z, _P]),
     "pbs_block_mask_to_csr": (c_int, [_P, _P, _P, _P, _I, _I, _I, _P]),
     "pbs_sparse_attn_workspace_bytes": (c_size_t, [_I] * 4),
-    "pbs_sparse_attn_fwd": (c_int, [_P] * 8 + [_I] * 7 + [_L] * 9 + [_F, _P, _P]),
-    "pbs_sparse_attn_fwd_optional_diagonal": (c_int, [_P] * 9 + [_I] * 6 + [_L] * 9 + [_F, _P, _P]),
+    "pbs_sparse_attn_fwd": (c_int, [_P] * 8 + [_I] * 7 + [_L] * 12 + [_F, _P, _P]),
+    "pbs_sparse_attn_fwd_optional_diagonal": (c_int, [_P] * 9 + [_I] * 6 + [_L] * 12 + [_F, _P, _P]),
     "pbs_unpermute": (c_int, [_P, _P, _P, _I, _I, _I, _I, _L, _L, _L, _P]),
     "pbs_rope_qk": (c_int, [_P] * 6 + [_I] * 5 + [_L] * 8 + [_P]),
     "pbs_identity_indices": (c_int, [_P, _I, _I, _P]),

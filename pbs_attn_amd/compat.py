@@ -154,12 +154,12 @@ def sparse_attention_on_block_mask(perm_Q, perm_K, perm_V, perm_O, perm_Q_indice
     k_orig = ops.unpermute(k.contiguous(), k_idx, torch.empty_like(k, memory_format=torch.contiguous_format))
     v_orig = ops.unpermute(v.contiguous(), v_idx, torch.empty_like(v, memory_format=torch.contiguous_format))
     pad_idx = torch.cat([k_idx, torch.arange(S, nb * block_size, dtype=torch.int32, device=dev).expand(B, H, -1)], dim=-1)
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(k_orig, v_orig, pad_idx.contiguous(), H, want_orig_vt=True, want_pooled=False)
+    perm_k, perm_vt, _ = ops.gather_kv(k_orig, v_orig, pad_idx.contiguous(), H, want_pooled=False)
     cols, cnt, missing = ops.block_mask_to_csr(block_mask.to(dev).expand(B, H, nb, nb), segment_size // block_size)
     if int(missing.item()) != 0:
         raise ValueError("block_mask leaves out blocks of a query block's own segment: the HIP attention kernel "
                          "always attends to the visible keys of the whole own segment (as pbs.py:209 arranges)")
-    out = ops.sparse_attn_fwd(perm_Q, perm_k, perm_vt, k_orig, orig_vt, cols, cnt, segment_size, 1.0 / (D ** 0.5))
+    out = ops.sparse_attn_fwd(perm_Q, perm_k, perm_vt, k_orig, v_orig, cols, cnt, segment_size, 1.0 / (D ** 0.5))
     perm_O.copy_(out)
     return perm_O
 

@@ -2,7 +2,7 @@
 //
 // What a query block attends to
 //   * the permuted K / V tiles of the selected key blocks of EARLIER segments (the visit list), no mask;
-//   * its own segment, read from the ORIGINAL K and the original-order transposed V: blocks
+//   * its own segment, read from the ORIGINAL K and V (the caller's tensors, in place): blocks
 //     first-of-segment .. query block, with the plain causal triangle on the last one (the diagonal block).
 //     A segment's permuted blocks hold the same keys as its original blocks and attention does not depend
 //     on key order, so this is the reference's "every block of the own segment, element mask original key
@@ -23,8 +23,9 @@
 //   visit lists (a few tiles per item) that is the difference between waiting for HBM three times per item
 //   and once.
 // Data layout
-//   K tile: 128 keys x 128 d row-major; V tile: stored TRANSPOSED in HBM by the gather kernel,
-//   128 d x 128 keys.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
+//   K tile: 128 keys x 128 d row-major; permuted V tile: stored TRANSPOSED in HBM by the gather kernel,
+//   128 d x 128 keys; V tile of an own segment: 128 keys x 128 d as in the caller's tensor, its MFMA fragments
+//   read with the transposing LDS read.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
 //   (row & 15): v_mfma fragment reads (row = lane % 32, 16 bytes) are bank-conflict free.
 // Math (transposed formulation, v_mfma_f32_32x32x16_bf16)
 //     S^T = K Q^T   (rows = keys, columns = queries)      O^T += V^T P^T   (rows = d, columns = queries)
@@ -54,16 +55,16 @@ struct AttnArgs {
   const uint16_t* pk;    // (B*Hq, nb*128, 128)  permuted K
   const uint16_t* pvt;   // (B*Hq, nb, 128, 128) permuted V blocks, transposed
   const uint16_t* k;     // original K at the KV heads, caller's strides
-  const uint16_t* ovt;   // (B*Hkv, nb, 128, 128) original-order V blocks, transposed
+  const uint16_t* v;     // original V at the KV heads, caller's strides
   const uint16_t* plist; // (B*Hq * npair, cap) merged visit lists
   int* queue;            // 8 work counters, one per XCD
   int cap;               // entries per list row (multiple of 8)
   uint16_t* o;
   int BH, Hq, Hkv, S, nb, bps;
-  uint32_t k_ss;   // key row stride in elements (< 2^22)
+  uint32_t k_ss, v_ss;   // key / value row strides in elements (< 2^22)
   int xcd_start[9];   // work items (head-major, long rows first) of XCD x: [xcd_start[x], xcd_start[x + 1])
   int interleave;     // 0, or 1 + log2(whole heads per XCD range) of a small launch whose tickets go pair-major (see ticket_item)
-  int64_t q_sb, q_sh, q_ss, k_sb, k_sh, o_sb, o_sh, o_ss;
+  int64_t q_sb, q_sh, q_ss, k_sb, k_sh, v_sb, v_sh, o_sb, o_sh, o_ss;
   float scale_log2;
 };
 
@@ -234,8 +235,8 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
 
   // base pointers of one head's tiles: permuted K, permuted V^T, original K rows, original-order V^T
   struct HeadBase {
-    const uint16_t *pk, *pvt, *korig, *ovt;
-    uint32_t k_ss;
+    const uint16_t *pk, *pvt, *korig, *vorig;
+    uint32_t k_ss, v_ss;
     int S;
   };
   auto head_base = [&](ArgsPtr ap, int bh_e) {
@@ -245,19 +246,20 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     hb.pk = ap->pk + (int64_t)bh_e * nb_e * BS * D;
     hb.pvt = ap->pvt + (int64_t)bh_e * nb_e * BS * D;
     hb.korig = ap->k + b_e * ap->k_sb + kvh * ap->k_sh;
-    hb.ovt = ap->ovt + (int64_t)(b_e * Hkv_e + kvh) * nb_e * BS * D;
+    hb.vorig = ap->v + b_e * ap->v_sb + kvh * ap->v_sh;
     hb.k_ss = ap->k_ss;
+    hb.v_ss = ap->v_ss;
     hb.S = ap->S;
     return hb;
   };
   // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf`
   auto stage_entry = [&](const HeadBase& hb, uint32_t e, uint32_t buf, int lane, uint32_t lane_off) {
     const int kb_e = (int)(e & ENT_KB);
-    if (e & ENT_ORIG) {
+    if (PBS_UNLIKELY(e & ENT_ORIG)) {
       // the lane id is formed afresh: offsets derived from the item's one are loop invariants that get hoisted out of
       // the tile loop and, when registers run out there, spilled and reloaded per tile
       stage_krows_async(hb.korig + (int64_t)kb_e * BS * hb.k_ss, hb.k_ss, hb.S - kb_e * BS, buf, wave, lane_id_here());
-      stage_tile_async(hb.ovt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+      stage_vrows_async(hb.vorig + (int64_t)kb_e * BS * hb.v_ss, hb.v_ss, hb.S - kb_e * BS, LDS_V0 + buf, wave, lane_id_here());
     } else {
       stage_tile_async(hb.pk + (int64_t)kb_e * BS * D, buf, wave, lane_off ^ k_copy_xor(wave));
       stage_tile_async(hb.pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
@@ -393,112 +395,139 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
           va[n] ^= 0x8000u;
         }
       };
-      for (int it = 0; it < n_tiles; ++it, next_buffers()) {
-        const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
-        const int kb = (int)(ent & ENT_KB);
+      // what every tile starts with: wait for its copies, hand over the buffers of the tile before, and request the
+      // copies of the tile after it (or, at the last tile, of the next item's first tile)
+      auto tile_head = [&](int it) {
         __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` (and of the next list) has landed
-        if (it == claim_it + 1) publish_and_fetch();
+        if (PBS_UNLIKELY(it == claim_it + 1)) publish_and_fetch();
         __syncthreads();                      // every share has; every wave is done with tile it - 1
-        if (it == claim_it + 1) adopt_next();
-        if (it == claim_it && wave == 0 && lane_id_here() == 0) claim = atomicAdd(PBS_ARGS()->queue + vic, 1);
-        if (it + 1 < n_tiles) stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
+        if (PBS_UNLIKELY(it == claim_it + 1)) adopt_next();
+        if (PBS_UNLIKELY(it == claim_it) && wave == 0 && lane_id_here() == 0) claim = atomicAdd(PBS_ARGS()->queue + vic, 1);
+        if (PBS_LIKELY(it + 1 < n_tiles)) stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
         else if (has_nxt && (careful_only || n_tiles >= 3))   // shorter items: after the loop, once the list has landed
           stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx ^ 0x8000u, lane, lane_off);
-        if (!(ent & use_bit) || !qb_valid) continue;
-        const bool masked = (ent & ENT_ORIG) && kb == qb;   // the diagonal block; other own-segment blocks lie before it
-
-        // careful: the first tile of a row, the redo pass, and masked tiles while some query has not seen a
-        // single key yet (its reference maximum is still -inf)
-        if (first && !masked && !careful_only) {
-          // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good
-          // enough reference to start the pipelined path (later keys move it up lazily)
-          first = false;
-          float mx[2] = {-INFINITY, -INFINITY};
+      };
+      // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good enough reference
+      // to start the pipelined path (later keys move it up lazily)
+      auto first_reference = [&]() {
+        first = false;
+        float mx[2] = {-INFINITY, -INFINITY};
+#pragma unroll
+        for (int T = 0; T < 2; ++T) {
+          f32x4 s0[2] = {(f32x4){0}, (f32x4){0}};
+#pragma unroll
+          for (int kd = 0; kd < 4; ++kd) {
+            const bf16x8 fk = ldsf(ka[kd] + T * 1024);
+#pragma unroll
+            for (int qg = 0; qg < 2; ++qg) s0[qg] = PBS_MFMA(fk, qf[qg][kd], s0[qg]);
+          }
+#pragma unroll
+          for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) mx[qg] = fmaxf(mx[qg], s0[qg][r]);
+        }
+#pragma unroll
+        for (int qg = 0; qg < 2; ++qg) m_ref[qg] = max_over_lane_groups(mx[qg]) * c_log2;
+        all_seen = true;
+      };
+      // careful tile: classic online softmax, one 32-key sub-tile at a time.  The redo pass, and a diagonal tile
+      // while some query has not seen a single key yet (its reference maximum is still -inf)
+      auto careful_tile = [&](uint32_t ent, bool masked) {
+        first = false;
+#pragma nounroll
+        for (int ks = 0; ks < 4; ++ks) {   // a real loop: the rare path stays small, in code and in registers
+          f32x4 s[2][2];   // [T][qg]
 #pragma unroll
           for (int T = 0; T < 2; ++T) {
-            f32x4 s0[2] = {(f32x4){0}, (f32x4){0}};
+            s[T][0] = (f32x4){0};
+            s[T][1] = (f32x4){0};
 #pragma unroll
             for (int kd = 0; kd < 4; ++kd) {
-              const bf16x8 fk = ldsf(ka[kd] + T * 1024);
+              const bf16x8 fk = ldsf(ka[kd] + T * 1024 + ks * 8192);
 #pragma unroll
-              for (int qg = 0; qg < 2; ++qg) s0[qg] = PBS_MFMA(fk, qf[qg][kd], s0[qg]);
-            }
-#pragma unroll
-            for (int qg = 0; qg < 2; ++qg)
-#pragma unroll
-              for (int r = 0; r < 4; ++r) mx[qg] = fmaxf(mx[qg], s0[qg][r]);
-          }
-#pragma unroll
-          for (int qg = 0; qg < 2; ++qg) m_ref[qg] = max_over_lane_groups(mx[qg]) * c_log2;
-          all_seen = true;
-          fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
-        } else if (first || careful_only || (masked && !all_seen)) {
-          // ---------------- careful tile: classic online softmax, one 32-key sub-tile at a time
-          first = false;
-#pragma nounroll
-          for (int ks = 0; ks < 4; ++ks) {   // a real loop: the rare path stays small, in code and in registers
-            f32x4 s[2][2];   // [T][qg]
-#pragma unroll
-            for (int T = 0; T < 2; ++T) {
-              s[T][0] = (f32x4){0};
-              s[T][1] = (f32x4){0};
-#pragma unroll
-              for (int kd = 0; kd < 4; ++kd) {
-                const bf16x8 fk = ldsf(ka[kd] + T * 1024 + ks * 8192);
-#pragma unroll
-                for (int qg = 0; qg < 2; ++qg) s[T][qg] = PBS_MFMA(fk, qf[qg][kd], s[T][qg]);
-              }
-            }
-            if (masked) {
-              const int ln = lane_id_here();   // keep the compares inside the tile (see fast_tile)
-              const int qrel8 = 32 * wq + (ln & 15) - 8 * (ln >> 4);
-#pragma unroll
-              for (int T = 0; T < 2; ++T)
-#pragma unroll
-                for (int qg = 0; qg < 2; ++qg)
-#pragma unroll
-                  for (int r = 0; r < 4; ++r)
-                    if (32 * ks + 4 * T + r - 16 * qg > qrel8) s[T][qg][r] = -INFINITY;
-            }
-            float alpha[2];
-            bf16x8 pf[2];
-#pragma unroll
-            for (int qg = 0; qg < 2; ++qg) {
-              float mx = fmaxf(fmaxf(s[0][qg][0], s[0][qg][1]), fmaxf(s[0][qg][2], s[0][qg][3]));
-              mx = fmaxf(mx, fmaxf(fmaxf(s[1][qg][0], s[1][qg][1]), fmaxf(s[1][qg][2], s[1][qg][3])));
-              mx = max_over_lane_groups(mx);
-              const float m_new = fmaxf(m_ref[qg], mx * c_log2);
-              const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-              alpha[qg] = __builtin_amdgcn_exp2f(m_ref[qg] - m_use);
-              m_ref[qg] = m_new;
-              float rs = 0.f;
-#pragma unroll
-              for (int e = 0; e < 8; ++e) {
-                const float pe = __builtin_amdgcn_exp2f(s[e >> 2][qg][e & 3] * c_log2 - m_use);
-                rs += pe;
-                pf[qg][e] = (__bf16)pe;
-              }
-              l_part[qg] = l_part[qg] * alpha[qg] + rs;
-            }
-            if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
-#pragma unroll
-              for (int dt = 0; dt < 8; ++dt)
-#pragma unroll
-                for (int qg = 0; qg < 2; ++qg)
-#pragma unroll
-                  for (int r = 0; r < 4; ++r) o[dt][qg][r] *= alpha[qg];
-            }
-#pragma unroll
-            for (int dt = 0; dt < 8; ++dt) {
-              const bf16x8 fv = ldsf((va[0] ^ (uint32_t)(ks << 6)) + dt * 4096);
-#pragma unroll
-              for (int qg = 0; qg < 2; ++qg) o[dt][qg] = PBS_MFMA(fv, pf[qg], o[dt][qg]);
+              for (int qg = 0; qg < 2; ++qg) s[T][qg] = PBS_MFMA(fk, qf[qg][kd], s[T][qg]);
             }
           }
-          all_seen = !__any(m_ref[0] == -INFINITY || m_ref[1] == -INFINITY);
-        } else {
-          if (masked) fast_tile<true, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
-          else fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+          if (masked) {
+            const int ln = lane_id_here();   // keep the compares inside the tile (see fast_tile)
+            const int qrel8 = 32 * wq + (ln & 15) - 8 * (ln >> 4);
+#pragma unroll
+            for (int T = 0; T < 2; ++T)
+#pragma unroll
+              for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                  if (32 * ks + 4 * T + r - 16 * qg > qrel8) s[T][qg][r] = -INFINITY;
+          }
+          float alpha[2];
+          bf16x8 pf[2];
+#pragma unroll
+          for (int qg = 0; qg < 2; ++qg) {
+            float mx = fmaxf(fmaxf(s[0][qg][0], s[0][qg][1]), fmaxf(s[0][qg][2], s[0][qg][3]));
+            mx = fmaxf(mx, fmaxf(fmaxf(s[1][qg][0], s[1][qg][1]), fmaxf(s[1][qg][2], s[1][qg][3])));
+            mx = max_over_lane_groups(mx);
+            const float m_new = fmaxf(m_ref[qg], mx * c_log2);
+            const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+            alpha[qg] = __builtin_amdgcn_exp2f(m_ref[qg] - m_use);
+            m_ref[qg] = m_new;
+            float rs = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float pe = __builtin_amdgcn_exp2f(s[e >> 2][qg][e & 3] * c_log2 - m_use);
+              rs += pe;
+              pf[qg][e] = (__bf16)pe;
+            }
+            l_part[qg] = l_part[qg] * alpha[qg] + rs;
+          }
+          if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt)
+#pragma unroll
+              for (int qg = 0; qg < 2; ++qg)
+#pragma unroll
+                for (int r = 0; r < 4; ++r) o[dt][qg][r] *= alpha[qg];
+          }
+#pragma unroll
+          for (int dt = 0; dt < 8; ++dt) {
+            const bf16x8 fv = (ent & ENT_ORIG)
+                                  ? ldsf_transposed(vrow_lane_addr(LDS_V0 + (va[0] & 0x8000u), lane_id_here()) + dt * 128 + ks * 8192)
+                                  : ldsf((va[0] ^ (uint32_t)(ks << 6)) + dt * 4096);
+#pragma unroll
+            for (int qg = 0; qg < 2; ++qg) o[dt][qg] = PBS_MFMA(fv, pf[qg], o[dt][qg]);
+          }
+        }
+        all_seen = !__any(m_ref[0] == -INFINITY || m_ref[1] == -INFINITY);
+      };
+      // The merged list holds the permuted tiles of earlier segments first, then the tiles of the own segments.  Each
+      // kind has a loop of its own, and so has the redo pass: a loop whose body updates the 64 accumulator registers
+      // on one path only keeps them in place, where several alternative tile bodies in one loop cost a copy of all of
+      // them per tile.
+      int it = 0;
+      if (PBS_UNLIKELY(careful_only)) {
+        for (; it < n_tiles; ++it, next_buffers()) {
+          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
+          tile_head(it);
+          if (!(ent & use_bit) || !qb_valid) continue;
+          careful_tile(ent, (ent & ENT_ORIG) && (int)(ent & ENT_KB) == qb);
+        }
+      } else {
+        for (; it < n_tiles; ++it, next_buffers()) {
+          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
+          if (PBS_UNLIKELY(ent & ENT_ORIG)) break;
+          tile_head(it);
+          if (PBS_UNLIKELY(!(ent & use_bit) || !qb_valid)) continue;
+          if (PBS_UNLIKELY(first)) first_reference();
+          fast_tile<false, PREFETCH_SLOTS, false>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+        }
+        for (; it < n_tiles; ++it, next_buffers()) {
+          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
+          tile_head(it);
+          if (!(ent & use_bit) || !qb_valid) continue;
+          const bool masked = (int)(ent & ENT_KB) == qb;   // the diagonal block; other own-segment blocks lie before it
+          if (first && !masked) first_reference();
+          if (first || (masked && !all_seen)) careful_tile(ent, masked);
+          else if (masked) fast_tile<true, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+          else fast_tile<false, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
         }
       }
       if (!careful_only && n_tiles < 3) {
@@ -625,58 +654,62 @@ extern "C" size_t pbs_sparse_attn_workspace_bytes(int B, int Hq, int S, int segm
   return 256 + (size_t)B * Hq * npair * cap * 2;
 }
 
-static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* v,
                               const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
                               int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                              float softmax_scale, const uint8_t* own_block_needed, void* workspace, void* stream);
+                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int64_t o_sb,
+                              int64_t o_sh, int64_t o_ss, float softmax_scale, const uint8_t* own_block_needed, void* workspace,
+                              void* stream);
 
-extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k,
-                                   const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B,
-                                   int Hq, int Hkv, int S, int head_dim, int block_size, int segment_size, int64_t q_sb,
-                                   int64_t q_sh, int64_t q_ss, int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb,
-                                   int64_t o_sh, int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
-  return sparse_attn_launch(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size,
-                            segment_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, nullptr,
+extern "C" int pbs_sparse_attn_fwd(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* v,
+                                   const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
+                                   int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
+                                   int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss,
+                                   int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
+  return sparse_attn_launch(q, perm_k, perm_vt, k, v, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size, segment_size,
+                            q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_scale, nullptr,
                             workspace, stream);
 }
 
 extern "C" int pbs_sparse_attn_fwd_optional_diagonal(const void* q, const void* perm_k, const void* perm_vt, const void* k,
-                                                     const void* orig_vt, const int32_t* csr_cols, const int32_t* csr_cnt,
+                                                     const void* v, const int32_t* csr_cols, const int32_t* csr_cnt,
                                                      const uint8_t* own_block_needed, void* out, int B, int Hq, int Hkv, int S,
                                                      int head_dim, int block_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                                                     int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh,
-                                                     int64_t o_ss, float softmax_scale, void* workspace, void* stream) {
+                                                     int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh,
+                                                     int64_t v_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss, float softmax_scale,
+                                                     void* workspace, void* stream) {
   PBS_REQUIRE(own_block_needed, "pbs_sparse_attn_fwd_optional_diagonal: null own_block_needed");
-  return sparse_attn_launch(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size,
-                            block_size, q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, own_block_needed,
-                            workspace, stream);
+  return sparse_attn_launch(q, perm_k, perm_vt, k, v, csr_cols, csr_cnt, out, B, Hq, Hkv, S, head_dim, block_size, block_size,
+                            q_sb, q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_scale,
+                            own_block_needed, workspace, stream);
 }
 
-static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* orig_vt,
+static int sparse_attn_launch(const void* q, const void* perm_k, const void* perm_vt, const void* k, const void* v,
                               const int32_t* csr_cols, const int32_t* csr_cnt, void* out, int B, int Hq, int Hkv, int S,
                               int head_dim, int block_size, int segment_size, int64_t q_sb, int64_t q_sh, int64_t q_ss,
-                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t o_sb, int64_t o_sh, int64_t o_ss,
-                              float softmax_scale, const uint8_t* own_block_needed, void* workspace, void* stream) {
-  PBS_REQUIRE(q && perm_k && perm_vt && k && orig_vt && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
+                              int64_t k_sb, int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int64_t o_sb,
+                              int64_t o_sh, int64_t o_ss, float softmax_scale, const uint8_t* own_block_needed, void* workspace,
+                              void* stream) {
+  PBS_REQUIRE(q && perm_k && perm_vt && k && v && csr_cols && csr_cnt && out, "pbs_sparse_attn_fwd: null tensor pointer");
   PBS_REQUIRE(workspace && ((uintptr_t)workspace % 256) == 0, "pbs_sparse_attn_fwd: workspace must be a 256-byte aligned device buffer of pbs_sparse_attn_workspace_bytes()");
   PBS_REQUIRE(head_dim == D && block_size == BS, "pbs_sparse_attn_fwd: head_dim and block_size must be 128 (got %d, %d)", head_dim, block_size);
   PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_sparse_attn_fwd: bad shape");
   PBS_REQUIRE(segment_size > 0 && segment_size % block_size == 0, "pbs_sparse_attn_fwd: segment_size must be a multiple of block_size");
   PBS_REQUIRE(segment_size / block_size <= 511, "pbs_sparse_attn_fwd: more than 511 blocks per segment");
   PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && o_sb % 8 == 0 && o_sh % 8 == 0 && o_ss % 8 == 0 &&
-                  k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0,
+                  k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_ss % 8 == 0,
               "pbs_sparse_attn_fwd: strides must keep rows 16-byte aligned");
   PBS_REQUIRE(k_ss >= D && k_ss < (1 << 22), "pbs_sparse_attn_fwd: key row stride %lld outside [128, 2^22)", (long long)k_ss);
+  PBS_REQUIRE(v_ss >= D && v_ss < (1 << 22), "pbs_sparse_attn_fwd: value row stride %lld outside [128, 2^22)", (long long)v_ss);
   PBS_REQUIRE(((uintptr_t)q % 16) == 0 && ((uintptr_t)out % 16) == 0 && ((uintptr_t)perm_k % 16) == 0 &&
-                  ((uintptr_t)perm_vt % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)orig_vt % 16) == 0,
+                  ((uintptr_t)perm_vt % 16) == 0 && ((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0,
               "pbs_sparse_attn_fwd: pointers must be 16-byte aligned");
   AttnArgs a;
   a.q = (const uint16_t*)q; a.pk = (const uint16_t*)perm_k; a.pvt = (const uint16_t*)perm_vt;
-  a.k = (const uint16_t*)k; a.ovt = (const uint16_t*)orig_vt;
+  a.k = (const uint16_t*)k; a.v = (const uint16_t*)v;
   a.o = (uint16_t*)out;
   a.BH = B * Hq; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS; a.bps = segment_size / block_size;
-  a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = (uint32_t)k_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
+  a.q_sb = q_sb; a.q_sh = q_sh; a.q_ss = q_ss; a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = (uint32_t)k_ss; a.v_sb = v_sb; a.v_sh = v_sh; a.v_ss = (uint32_t)v_ss; a.o_sb = o_sb; a.o_sh = o_sh; a.o_ss = o_ss;
   a.scale_log2 = softmax_scale * 1.4426950408889634f;
   PBS_REQUIRE(a.nb <= 4096, "pbs_sparse_attn_fwd: more than 4096 blocks per sequence (%d)", a.nb);
   // eight ranges of equal estimated work: the row pair p of a head costs about p + 1 (causal length)

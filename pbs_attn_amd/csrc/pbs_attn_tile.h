@@ -4,6 +4,12 @@
 #pragma once
 #include "pbs_common.h"
 
+// branch hints: they decide which side of a branch is laid out as the fall-through.  A taken branch refills the
+// wave's instruction buffer, and in the tile loop all eight waves of a workgroup take it at about the same time with
+// the matrix pipes idle, so the common path of that loop has to be the straight one.
+#define PBS_LIKELY(x) __builtin_expect(!!(x), 1)
+#define PBS_UNLIKELY(x) __builtin_expect(!!(x), 0)
+
 namespace {
 
 
@@ -44,6 +50,13 @@ __device__ __forceinline__ int lane_id_here() {
 // (= i: sixteen chunks, no bank conflict); rows of a V^T tile are d and the lanes take consecutive rows: row & 15.
 __device__ __forceinline__ int k_row_hash(int row) { return (row & 3) | (((row >> 3) & 3) << 2); }
 
+// A tile of V rows taken from the caller's tensor (a query block's own segment) is not transposed on the way in.  Its
+// fragments are read with the transposing LDS read (ds_read_b64_tr_b16: lane l of a group of 16 hands in the address of
+// four consecutive d of key (l / 4), and receives, for d = l, the four keys), two reads per fragment.  Four rows (keys
+// 4 m + 0..3) share 1024 bytes of LDS, 32-byte piece p (d = 16 p .. 16 p + 15) of row 4 m + e at m * 1024 + p * 128 +
+// e * 32: a group's four keys x 32 bytes are 128 consecutive bytes (no bank conflict), the d tile, the sub-tile and the
+// key half of a read are constant offsets from one address per lane, and one copy instruction (1024 bytes of LDS)
+// reads four whole rows.
 // the copy of a K tile fetches chunk (l & 15) ^ k_row_hash(row) where async_lane_offset has (l & 15) ^ (row & 15), row =
 // 4 wave + (l >> 4) + 32 n: the two differ by a wave-uniform XOR of the byte offset
 __device__ __forceinline__ uint32_t k_copy_xor(int wave) { return (uint32_t)(((wave & 3) ^ ((wave >> 1) & 3)) << 6); }
@@ -78,7 +91,7 @@ __device__ __forceinline__ void stage_tile_async(const uint16_t* src, uint32_t l
   }
 }
 
-// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride (the LDS layout of a K tile, k_row_hash below).  Rows
+// K tile of the ORIGINAL tensor: 128 rows at the caller's row stride, chunk index XOR k_row_hash of the row.  Rows
 // past the end of the sequence re-read the last valid row: their keys lie after every query and are masked.
 __device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t row_stride, int rows_valid, uint32_t lds_byte,
                                                   int wave, int lane) {
@@ -87,11 +100,42 @@ __device__ __forceinline__ void stage_krows_async(const uint16_t* src, uint32_t 
   const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
   const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
   const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
-  // lane l of wave w fetches chunk (l & 15) ^ (row & 15) of row 4 w + 32 n + (l >> 4); offsets fit 32 bits
-  // (row stride < 2^22 elements, checked on the host)
+  // lane l of wave w fetches chunk (l & 15) ^ hash(row) of row 4 w + 32 n + (l >> 4) (the hash does not depend on n);
+  // offsets fit 32 bits (row stride < 2^22 elements, checked on the host)
   const uint32_t r0 = (uint32_t)(4 * wave + (lane >> 4));
   const uint32_t c16 = (uint32_t)(((lane & 15) ^ k_row_hash((int)r0)) * 16);
-  if (rows_valid >= BS) {
+  if (PBS_LIKELY(rows_valid >= BS)) {
+    const uint32_t voff = r0 * row_stride * 2u + c16;
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const uint64_t base = srcu + (uint64_t)n * (64u * row_stride);
+      register uint32_t m0v asm("m0") = lds0 + n * 8192;
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(base) : "memory");
+    }
+  } else {
+#pragma unroll
+    for (int n = 0; n < 4; ++n) {
+      const uint32_t row = min(r0 + 32u * n, (uint32_t)(rows_valid - 1));
+      const uint32_t voff = row * row_stride * 2u + c16;
+      register uint32_t m0v asm("m0") = lds0 + n * 8192;
+      asm volatile("s_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(m0v), "v"(voff), "s"(srcu) : "memory");
+    }
+  }
+}
+
+// V tile of the ORIGINAL tensor in the layout above: wave w, instruction n copy rows 4 w + 32 n + 0..3 like the K copy;
+// lane l takes row (l >> 1) & 3 of them and the 16-byte chunk 2 (l >> 3) + (l & 1).  Rows past the end of the sequence
+// re-read the last valid row.
+__device__ __forceinline__ void stage_vrows_async(const uint16_t* src, uint32_t row_stride, int rows_valid, uint32_t lds_byte,
+                                                  int wave, int lane) {
+  const uint32_t lds0 = (uint32_t)__builtin_amdgcn_readfirstlane((int)(lds_byte + wave * 1024));
+  const uint64_t src0 = (uint64_t)(uintptr_t)src;
+  const uint32_t src_lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)src0);
+  const uint32_t src_hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(src0 >> 32));
+  const uint64_t srcu = ((uint64_t)src_hi << 32) | (uint64_t)src_lo;
+  const uint32_t r0 = (uint32_t)(4 * wave + ((lane >> 1) & 3));
+  const uint32_t c16 = (uint32_t)((2 * (lane >> 3) + (lane & 1)) * 16);
+  if (PBS_LIKELY(rows_valid >= BS)) {
     const uint32_t voff = r0 * row_stride * 2u + c16;
 #pragma unroll
     for (int n = 0; n < 4; ++n) {
@@ -118,6 +162,24 @@ __device__ __forceinline__ bf16x8 ldsf(uint32_t byte_addr) {
 // B, each with k = 8 (l / 16) + 0..7, and of D column l % 16, rows 4 (l / 16) + 0..3.  On normally distributed
 // operands the chip sustains about 11 % more FLOP/s with this shape than with 32x32x16 (it moves half the
 // accumulator registers per FLOP and holds a higher clock inside its power limit).
+// V^T fragment (16 d x 32 keys of a sub-tile) out of a tile copied by stage_vrows_async: addr = this lane's address
+// for the fragment's d tile and sub-tile; keys 8 g + 0..3 at addr, 8 g + 4..7 in the next four rows (1024 bytes further)
+typedef __attribute__((ext_vector_type(4))) short s16x4;
+__device__ __forceinline__ bf16x8 ldsf_transposed(uint32_t addr) {
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds_u8*)(uintptr_t)addr);
+  const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(lds_u8*)(uintptr_t)(addr + 1024));
+  typedef __attribute__((ext_vector_type(8))) short s16x8;
+  const s16x8 both = {lo[0], lo[1], lo[2], lo[3], hi[0], hi[1], hi[2], hi[3]};
+  return __builtin_bit_cast(bf16x8, both);
+}
+// this lane's address of the fragment of sub-tile 0, d tile 0 in the tile whose buffer starts at LDS byte offset
+// v_buf; d tile dt: + dt * 128, sub-tile ks: + ks * 8192
+__device__ __forceinline__ uint32_t vrow_lane_addr(uint32_t v_buf, int lane) {
+  const int l16 = lane & 15, g = lane >> 4;
+  return v_buf + (uint32_t)(g * 2048 + (l16 >> 2) * 32 + (l16 & 3) * 8);
+}
+
 #define PBS_MFMA(a, b, c) __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0)
 
 // lane ^ 16: with xhalf_f32 (lane ^ 32) it reaches the four lanes that share a query column
@@ -141,7 +203,9 @@ __device__ __forceinline__ float sum_over_lane_groups(float v) {
 // fragments of sub-tile ks (d tile 0) in the tile's buffers: held in registers and switched between the two buffers
 // once per tile, so that a fragment read needs no address arithmetic (a vector instruction per read is a tenth of
 // the pipeline's vector work, and vector work overlaps only a third of a matrix instruction's time).
-template <bool MASKED, int PF>
+// V_ROWS: the tile's V is a tile of the caller's tensor, copied by stage_vrows_async, and its fragments come from
+// transposing reads; otherwise it is a transposed (V^T) tile and they are plain 16-byte reads.
+template <bool MASKED, int PF, bool V_ROWS>
 __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2][4], const uint32_t (&ka)[4],
                                           const uint32_t (&va)[4], float c_log2, float (&m_ref)[2],
                                           float (&l_part)[2], bool& poisoned, int wq) {
@@ -154,6 +218,8 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
     qrel8 = 32 * wq + (ln & 15) - 8 * (ln >> 4);
   }
   const float negm[2] = {-m_ref[0], -m_ref[1]};
+  uint32_t vr = 0;
+  if (V_ROWS) vr = vrow_lane_addr(LDS_V0 + (va[0] & 0x8000u), lane_id_here());   // va[] carries the buffer switch in bit 15
   float rsum[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
   f32x4 sacc[2][2][2];     // [sub-tile parity][T][qg]
   bf16x8 pbuf[2][2];       // [sub-tile parity][qg]
@@ -167,7 +233,13 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
     {   // fragment reads for slot n + PF
       const int m = n + PF, mstep = m >> 3, mt = m & 7;
       if (m < 48 && mstep <= 3) frk[m % R] = ldsf(ka[mt & 3] + (mt >> 2) * 1024 + mstep * 8192);
-      if (m < 48 && mstep >= 2) frv[m % R] = ldsf(va[mstep - 2] + mt * 4096);
+      if (m < 48 && mstep >= 2) {
+        if (V_ROWS) {
+          frv[m % R] = ldsf_transposed(vr + mt * 128 + (mstep - 2) * 8192);
+        } else {
+          frv[m % R] = ldsf(va[mstep - 2] + mt * 4096);
+        }
+      }
     }
     // the reads go out before this slot's matrix instructions: left to the scheduler they sink behind them
     // (their address is formed in the slot) and the fragments arrive a slot late
@@ -207,7 +279,7 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
   l_part[1] += rs[1];
   // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
   // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
-  if (__any(rs[0] > 16384.0f || rs[1] > 16384.0f)) {
+  if (PBS_UNLIKELY(__any(rs[0] > 16384.0f || rs[1] > 16384.0f))) {
 #pragma unroll
     for (int qg = 0; qg < 2; ++qg) {
       const float big = max_over_lane_groups(rs[qg]);

@@ -5,9 +5,6 @@
 //   perm_vt (B, Hq, nb, 128, 128)  V block TRANSPOSED: [d][key in block] -- the
 //                                  layout the attention kernel feeds to MFMA
 //   pooled_k(B, Hq, nb, 128)       bf16 mean (fp32 accumulate / 128) or max
-//   orig_vt (B, Hkv, nb, 128, 128) V blocks in ORIGINAL order, transposed the same way and zero past S
-//                                  (the attention kernel reads a query block's own segment un-permuted);
-//                                  produced by B*Hkv extra grid rows of the same launch
 // A 256-byte source row is read by 16 lanes x 16 bytes; K/V may be stored at
 // the KV-head count (query head h reads KV head h / G).
 // The same kernel runs in two reduced forms so that a caller can gather only what the attention will read:
@@ -32,7 +29,6 @@ struct GatherArgs {
   uint16_t* perm_k;
   uint16_t* perm_vt;
   uint16_t* pooled_k;
-  uint16_t* orig_vt;
   uint8_t* needed;     // (B*Hq, nb) or null: filter (full form), cleared (pooling-only form)
   int B, Hq, Hkv, S, nb;
   int64_t k_sb, k_sh, k_ss, v_sb, v_sh, v_ss;
@@ -41,19 +37,17 @@ struct GatherArgs {
 
 template <bool POOL_ONLY>
 __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float (&pool)[16][D], int kb, int grid_row) {
-  const bool orig = !POOL_ONLY && grid_row >= a.B * a.Hq;   // extra grid rows: V of a KV head in original order
-  const int bh = orig ? grid_row - a.B * a.Hq : grid_row;
+  const int bh = grid_row;
   if (POOL_ONLY) {
     if (a.needed && threadIdx.x == 0) a.needed[(int64_t)bh * a.nb + kb] = 0;
-  } else if (!orig && a.needed && a.needed[(int64_t)bh * a.nb + kb] == 0) {
+  } else if (a.needed && a.needed[(int64_t)bh * a.nb + kb] == 0) {
     return;
   }
-  const int heads = orig ? a.Hkv : a.Hq;
-  const int b = bh / heads, h = bh % heads, kvh = orig ? h : h / (a.Hq / a.Hkv);
+  const int b = bh / a.Hq, h = bh % a.Hq, kvh = h / (a.Hq / a.Hkv);
   const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;  // row group, 16-byte chunk
   const uint16_t* ksrc = a.k + b * a.k_sb + kvh * a.k_sh;
   const uint16_t* vsrc = a.v + b * a.v_sb + kvh * a.v_sh;
-  const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS + kb * BS;   // not read for the extra rows
+  const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS + kb * BS;
   uint16_t* kdst = a.perm_k + ((int64_t)bh * a.nb + kb) * BS * D;
 
   float acc[8];
@@ -66,11 +60,11 @@ __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float 
     const int pos = kb * BS + i;
     u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
     if (pos < a.S) {
-      const int src = orig ? pos : idx[i];
-      if (!orig) kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
+      const int src = idx[i];
+      kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
       if (!POOL_ONLY) vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
     }
-    if (!POOL_ONLY && !orig) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
+    if (!POOL_ONLY) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const float lo = bf16_bits_to_f32(kv[e] & 0xffffu), hi = bf16_bits_to_f32(kv[e] >> 16);
@@ -89,7 +83,7 @@ __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float 
   for (int e = 0; e < 8; ++e) pool[rg][c * 8 + e] = acc[e];
   __syncthreads();
 
-  if (threadIdx.x < D && !orig && a.pooled_k) {
+  if (threadIdx.x < D && a.pooled_k) {
     float s = pool[0][threadIdx.x];
     for (int r = 1; r < 16; ++r) s = a.pool_max ? fmaxf(s, pool[r][threadIdx.x]) : s + pool[r][threadIdx.x];
     if (!a.pool_max) s = s / (float)BS;
@@ -98,7 +92,7 @@ __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float 
 
   if (POOL_ONLY) return;
   // transposed write-out: thread (d, key group of 8) -> 16 bytes of row d
-  uint16_t* vdst = (orig ? a.orig_vt : a.perm_vt) + ((int64_t)bh * a.nb + kb) * D * BS;
+  uint16_t* vdst = a.perm_vt + ((int64_t)bh * a.nb + kb) * D * BS;
 #pragma unroll
   for (int pass = 0; pass < 8; ++pass) {
     const int d = pass * 16 + rg;
@@ -184,7 +178,7 @@ __global__ __launch_bounds__(256) void pool_qk_kernel(GatherArgs a, PoolQArgs p)
 }  // namespace
 
 extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_indices, void* perm_k, void* perm_vt,
-                             void* pooled_k, void* orig_vt, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
+                             void* pooled_k, int B, int Hq, int Hkv, int S, int head_dim, int block_size, int64_t k_sb,
                              int64_t k_sh, int64_t k_ss, int64_t v_sb, int64_t v_sh, int64_t v_ss, int key_pool_max,
                              const uint8_t* block_needed, void* stream) {
   PBS_REQUIRE(k && v && key_indices && perm_k && perm_vt, "pbs_gather_kv: null tensor pointer");
@@ -193,17 +187,15 @@ extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_in
   PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_ss % 8 == 0,
               "pbs_gather_kv: strides must keep rows 16-byte aligned");
   PBS_REQUIRE(((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0, "pbs_gather_kv: pointers must be 16-byte aligned");
-  PBS_REQUIRE(B * (Hq + Hkv) <= 65535, "pbs_gather_kv: too many heads");
+  PBS_REQUIRE(B * Hq <= 65535, "pbs_gather_kv: too many heads");
   GatherArgs a;
   a.k = (const uint16_t*)k; a.v = (const uint16_t*)v; a.idx = key_indices;
   a.perm_k = (uint16_t*)perm_k; a.perm_vt = (uint16_t*)perm_vt; a.pooled_k = (uint16_t*)pooled_k;
-  a.orig_vt = (uint16_t*)orig_vt;
   a.needed = const_cast<uint8_t*>(block_needed);
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss; a.v_sb = v_sb; a.v_sh = v_sh; a.v_ss = v_ss;
   a.pool_max = key_pool_max;
-  // orig_vt may be null: then only the permuted outputs are produced; pooled_k may be null: no pooling
-  hipLaunchKernelGGL(gather_kv_kernel<false>, dim3(a.nb, B * Hq + (orig_vt ? B * Hkv : 0)), dim3(256), 0, (hipStream_t)stream, a);
+  hipLaunchKernelGGL(gather_kv_kernel<false>, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_gather_kv");
 }
 

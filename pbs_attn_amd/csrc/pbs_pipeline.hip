@@ -12,7 +12,7 @@ __global__ void identity_indices_kernel(int32_t* idx, int S_pad, int64_t total) 
 }
 
 struct Layout {
-  size_t scores, score_ws, idx, perm_k, perm_vt, orig_vt, pooled_k, pooled_q, probs, cols, cnt, needed, select_ws, attn_ws, total;
+  size_t scores, score_ws, idx, perm_k, perm_vt, pooled_k, pooled_q, probs, cols, cnt, needed, select_ws, attn_ws, total;
 };
 
 size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -29,7 +29,6 @@ Layout make_layout(int B, int Hq, int Hkv, int S, int D, int block_size, int seg
   L.idx = take(rows * s_pad * 4);
   L.perm_k = take(rows * s_pad * D * 2);
   L.perm_vt = take(rows * s_pad * D * 2);
-  L.orig_vt = take((size_t)B * Hkv * s_pad * D * 2);
   L.pooled_k = take(rows * nb * D * 2);
   L.pooled_q = take(rows * nb * D * 2);
   L.probs = take(rows * nb * nb * 4);
@@ -109,7 +108,7 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
   // (Every candidate selected: everything is visited, one full gather.)
   uint8_t* needed = threshold_is_int_one ? nullptr : w + L.needed;
   if (threshold_is_int_one) {
-    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, w + L.orig_vt, B, Hq, Hkv,
+    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, B, Hq, Hkv,
                             S, head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, nullptr, stream))) return rc;
   } else {
     if ((rc = pbs_pool_blocks(q, k, (const int32_t*)(w + L.idx), w + L.pooled_q, w + L.pooled_k, needed, B, Hq, Hkv, S,
@@ -130,10 +129,11 @@ extern "C" int pbs_prefill_attn_fwd(const void* q, const void* k, const void* v,
                               nullptr, nullptr, (int32_t*)(w + L.cols), (int32_t*)(w + L.cnt), needed, w + L.select_ws,
                               L.attn_ws - L.select_ws, stream))) return rc;
   if (!threshold_is_int_one) {
-    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, w + L.orig_vt, B, Hq, Hkv,
+    if ((rc = pbs_gather_kv(k, v, (const int32_t*)(w + L.idx), w + L.perm_k, w + L.perm_vt, nullptr, B, Hq, Hkv,
                             S, head_dim, block_size, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, key_pool_max, needed, stream))) return rc;
   }
-  return pbs_sparse_attn_fwd(q, w + L.perm_k, w + L.perm_vt, k, w + L.orig_vt, (const int32_t*)(w + L.cols),
+  return pbs_sparse_attn_fwd(q, w + L.perm_k, w + L.perm_vt, k, v, (const int32_t*)(w + L.cols),
                              (const int32_t*)(w + L.cnt), out, B, Hq, Hkv, S, head_dim, block_size, segment_size, q_sb,
-                             q_sh, q_ss, k_sb, k_sh, k_ss, o_sb, o_sh, o_ss, softmax_scale, w + L.attn_ws, stream);
+                             q_sh, q_ss, k_sb, k_sh, k_ss, v_sb, v_sh, v_ss, o_sb, o_sh, o_ss, softmax_scale, w + L.attn_ws,
+                             stream);
 }

@@ -19,7 +19,9 @@ double pbs_mfma_probe_flop(int iters);
  * per workgroup and tile, 8.389 MFLOP each) out of LDS, with the kernel's barrier per tile and, if `with_copies`,
  * its asynchronous copies of the next tile (64 KB from a ring of `n_src_tiles` >= 2 K / V^T tile pairs of 65536
  * bytes each at `tiles`, whose first 32 KB also serve as the queries) -- no visit lists, no write-out.  `sink`
- * takes 256 * 512 floats; `clocks` receives workgroup 0's shader-clock ticks and 100 MHz ticks.  Time the launch
+ * takes 256 * 512 floats; `clocks` receives workgroup 0's shader-clock ticks and 100 MHz ticks.  `with_copies`
+ * bit 1 handles the tiles as a tile of the query block's own segment is handled: K and V copied row by row, the V
+ * fragments formed by transposing reads.  Time the launch
  * with events: the same cycles per tile on every input, but on data the clock drops with the power limit. */
 int pbs_attn_tile_probe(const void* tiles, int n_src_tiles, int iters, int with_copies, float* sink,
                         unsigned long long* clocks, void* stream);

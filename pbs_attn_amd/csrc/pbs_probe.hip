@@ -72,7 +72,10 @@ namespace {
 // ---- measurement aid: the tile pipeline alone.  Every workgroup runs `iters` unmasked fast tiles out of its two
 // LDS buffer pairs with the kernel's per-tile barrier and, if asked, the kernel's 64 KB of copies per tile (from a
 // ring of `n_src` K / V^T tile pairs), without lists, items, write-out or rare paths: what the schedule of
-// fast_tile sustains by itself.  Workgroup 0 reports its shader-clock and 100 MHz ticks.
+// fast_tile sustains by itself.  V_ROWS: the tiles are handled as the kernel handles a tile of the query block's own
+// segment (K and V copied row by row, V fragments by transposing reads).  Workgroup 0 reports its shader-clock and
+// 100 MHz ticks.
+template <bool V_ROWS>
 __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __restrict__ tiles, int n_src, int iters, int with_copies,
                                                             float* __restrict__ sink, unsigned long long* __restrict__ clocks) {
   extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
@@ -111,8 +114,13 @@ __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __re
     __syncthreads();
     if (with_copies) {
       const uint16_t* src = tiles + (size_t)((it * 7 + (int)blockIdx.x / 8) % n_src) * (2 * BS * D);
-      stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off ^ k_copy_xor(wave));
-      stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+      if (V_ROWS) {
+        stage_krows_async(src, D, BS, bufx ^ 0x8000u, wave, lane_id_here());
+        stage_vrows_async(src + BS * D, D, BS, LDS_V0 + (bufx ^ 0x8000u), wave, lane_id_here());
+      } else {
+        stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off ^ k_copy_xor(wave));
+        stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+      }
     }
     uint32_t ka[4], va[4];
 #pragma unroll
@@ -120,7 +128,7 @@ __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __re
       ka[n] = koff0 ^ (uint32_t)(n << 6) ^ bufx;
       va[n] = voff0 ^ (uint32_t)(n << 6) ^ bufx;
     }
-    fast_tile<false, PREFETCH_SLOTS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wave & 3);
+    fast_tile<false, PREFETCH_SLOTS, V_ROWS>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wave & 3);
   }
   __builtin_amdgcn_s_waitcnt(0x0f70);
   const unsigned long long c1 = __builtin_amdgcn_s_memtime(), r1 = __builtin_amdgcn_s_memrealtime();
@@ -144,12 +152,18 @@ extern "C" int pbs_attn_tile_probe(const void* tiles, int n_src_tiles, int iters
                                    unsigned long long* clocks, void* stream) {
   PBS_REQUIRE(tiles && sink && clocks && iters > 0 && n_src_tiles >= 2, "pbs_attn_tile_probe: bad arguments");
   PBS_REQUIRE(((uintptr_t)tiles % 16) == 0, "pbs_attn_tile_probe: tiles must be 16-byte aligned");
-  hipError_t attr = hipFuncSetAttribute((const void*)tile_probe_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
+  const bool v_rows = (with_copies & 2) != 0;
+  const void* kernel = v_rows ? (const void*)tile_probe_kernel<true> : (const void*)tile_probe_kernel<false>;
+  hipError_t attr = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)LDS_TOTAL);
   if (attr != hipSuccess) {
     pbs_set_error("pbs_attn_tile_probe: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
     return (int)attr;
   }
-  hipLaunchKernelGGL(tile_probe_kernel, dim3(256), dim3(512), LDS_TOTAL, (hipStream_t)stream, (const uint16_t*)tiles, n_src_tiles,
-                     iters, with_copies, sink, clocks);
+  if (v_rows)
+    hipLaunchKernelGGL(tile_probe_kernel<true>, dim3(256), dim3(512), LDS_TOTAL, (hipStream_t)stream, (const uint16_t*)tiles,
+                       n_src_tiles, iters, with_copies & 1, sink, clocks);
+  else
+    hipLaunchKernelGGL(tile_probe_kernel<false>, dim3(256), dim3(512), LDS_TOTAL, (hipStream_t)stream, (const uint16_t*)tiles,
+                       n_src_tiles, iters, with_copies & 1, sink, clocks);
   return pbs_check_launch("pbs_attn_tile_probe");
 }

@@ -39,8 +39,7 @@ def MeanPooling_prefill(
     s_pad = (q_len + block_size - 1) // block_size * block_size
     idx = torch.arange(s_pad, dtype=torch.int32, device=query_states.device).view(1, 1, -1)
     idx = idx.expand(batch_size, num_q_heads, -1).contiguous()
-    perm_k, perm_vt, pooled_k, orig_vt = ops.gather_kv(key_states, value_states, idx, num_q_heads, "mean",
-                                                       want_orig_vt=True)
+    perm_k, perm_vt, pooled_k = ops.gather_kv(key_states, value_states, idx, num_q_heads, "mean")
     pooled_q = ops.pool_q(query_states, "mean")
     scores = ops.block_logits_softmax(pooled_q, pooled_k, 1, causal_candidates=True)
     # MeanPooling.py:50 hands the threshold to select_blocks as it is: there is no "int 1 = everything" rule here
@@ -55,7 +54,7 @@ def MeanPooling_prefill(
         # selection mask says where
         fin = sel   # the selection with the forced first column, without the forced diagonal
         own = fin.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
-    out = ops.sparse_attn_fwd(query_states, perm_k, perm_vt, key_states, orig_vt, cols, cnt, block_size, own_block_needed=own)
+    out = ops.sparse_attn_fwd(query_states, perm_k, perm_vt, key_states, value_states, cols, cnt, block_size, own_block_needed=own)
     if return_masks:
         return out, dict(block_attn_scores=scores, block_mask=fin, csr_cnt=cnt)
     return out

@@ -87,9 +87,8 @@ def segment_argsort(scores, seq_len, segment_size, block_size=BLOCK):
     return idx
 
 
-def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False, block_needed=None, want_pooled=True):
-    """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128), pooled_k (B, Hq, nb, D) and, with
-    ``want_orig_vt``, orig_vt (B, Hkv, nb, D, 128): the V blocks in original order, transposed.
+def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", block_needed=None, want_pooled=True):
+    """Returns perm_k (B, Hq, S_pad, D), perm_vt (B, Hq, nb, D, 128) and pooled_k (B, Hq, nb, D).
     ``block_needed`` ((B, Hq, nb) uint8, from ``select_blocks(..., block_needed=...)``) restricts the gather to
     the blocks whose byte is set: the other tiles of perm_k / perm_vt stay uninitialised.  ``want_pooled=False``
     returns None for pooled_k."""
@@ -105,16 +104,13 @@ def gather_kv(k, v, idx, num_q_heads, key_pool_mode="mean", want_orig_vt=False, 
     perm_k = torch.empty((B, Hq, nb * BLOCK, D), dtype=k.dtype, device=k.device)
     perm_vt = torch.empty((B, Hq, nb, D, BLOCK), dtype=k.dtype, device=k.device)
     pooled_k = torch.empty((B, Hq, nb, D), dtype=k.dtype, device=k.device) if want_pooled else None
-    orig_vt = torch.empty((B, Hkv, nb, D, BLOCK), dtype=k.dtype, device=k.device) if want_orig_vt else None
     if block_needed is not None:
         assert block_needed.shape == (B, Hq, nb) and block_needed.dtype == torch.uint8 and block_needed.is_contiguous()
-    _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k), _ptr(orig_vt),
+    _lib.check(lib.pbs_gather_kv(_ptr(k), _ptr(v), _ptr(idx), _ptr(perm_k), _ptr(perm_vt), _ptr(pooled_k),
                                  B, Hq, Hkv, S, D, BLOCK, k.stride(0), k.stride(1), k.stride(2),
                                  v.stride(0), v.stride(1), v.stride(2), int(key_pool_mode == "max"),
                                  _ptr(block_needed), _stream()),
                "pbs_gather_kv")
-    if want_orig_vt:
-        return perm_k, perm_vt, pooled_k, orig_vt
     return perm_k, perm_vt, pooled_k
 
 
@@ -249,15 +245,15 @@ def block_mask_to_csr(block_mask, blocks_per_segment):
     return cols, cnt, missing
 
 
-def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None,
+def sparse_attn_fwd(q, perm_k, perm_vt, k, v, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None,
                     own_block_needed=None):
     """Attention of every query block over the permuted tiles listed in the CSR (earlier segments) and
-    over the causal part of its own segment, read from the original ``k`` (B, Hkv or Hq, S, D) and
-    ``orig_vt``.  ``own_block_needed`` ((B, Hq, nb) uint8, one-block segments only) makes the diagonal block
+    over the causal part of its own segment, read in place from the original ``k`` and ``v`` (B, Hkv or Hq, S, D).
+    ``own_block_needed`` ((B, Hq, nb) uint8, one-block segments only) makes the diagonal block
     optional per query block."""
-    _check_bf16_cuda(q, perm_k, perm_vt, k, orig_vt)
+    _check_bf16_cuda(q, perm_k, perm_vt, k, v)
     lib = _lib.load()
-    q, k = _rows16(q), _rows16(k)
+    q, k, v = _rows16(q), _rows16(k), _rows16(v)
     B, Hq, S, D = q.shape
     Hkv = k.shape[1]
     if softmax_scale is None:
@@ -265,25 +261,25 @@ def sparse_attn_fwd(q, perm_k, perm_vt, k, orig_vt, csr_cols, csr_cnt, segment_s
     if out is None:
         out = torch.empty((B, Hq, S, D), dtype=q.dtype, device=q.device)
     nb = (S + BLOCK - 1) // BLOCK
-    assert perm_k.is_contiguous() and perm_vt.is_contiguous() and orig_vt.is_contiguous()
+    assert perm_k.is_contiguous() and perm_vt.is_contiguous()
     assert perm_k.shape == (B, Hq, nb * BLOCK, D) and perm_vt.shape == (B, Hq, nb, D, BLOCK)
-    assert k.shape == (B, Hkv, S, D) and orig_vt.shape == (B, Hkv, nb, D, BLOCK)
+    assert k.shape == (B, Hkv, S, D) and v.shape == (B, Hkv, S, D)
     assert csr_cols.is_contiguous() and csr_cnt.is_contiguous()
     assert csr_cols.shape == (B, Hq, nb, nb) and csr_cnt.shape == (B, Hq, nb)
     ws = torch.empty(max(lib.pbs_sparse_attn_workspace_bytes(B, Hq, S, segment_size), 256), dtype=torch.uint8, device=q.device)
+    strides = (q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2), v.stride(0), v.stride(1), v.stride(2),
+               out.stride(0), out.stride(1), out.stride(2))
     if own_block_needed is not None:
         if segment_size != BLOCK:
             raise ValueError("own_block_needed: only for one-block segments (segment_size == block_size)")
         assert own_block_needed.shape == (B, Hq, nb) and own_block_needed.dtype == torch.uint8 and own_block_needed.is_contiguous()
         _lib.check(lib.pbs_sparse_attn_fwd_optional_diagonal(
-            _ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols), _ptr(csr_cnt), _ptr(own_block_needed),
-            _ptr(out), B, Hq, Hkv, S, D, BLOCK, q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-            out.stride(0), out.stride(1), out.stride(2), softmax_scale, _ptr(ws), _stream()), "pbs_sparse_attn_fwd_optional_diagonal")
+            _ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(v), _ptr(csr_cols), _ptr(csr_cnt), _ptr(own_block_needed),
+            _ptr(out), B, Hq, Hkv, S, D, BLOCK, *strides, softmax_scale, _ptr(ws), _stream()), "pbs_sparse_attn_fwd_optional_diagonal")
         return out
-    _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(orig_vt), _ptr(csr_cols),
-                                       _ptr(csr_cnt), _ptr(out), B, Hq, Hkv, S, D, BLOCK, segment_size,
-                                       q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-                                       out.stride(0), out.stride(1), out.stride(2), softmax_scale, _ptr(ws), _stream()),
+    _lib.check(lib.pbs_sparse_attn_fwd(_ptr(q), _ptr(perm_k), _ptr(perm_vt), _ptr(k), _ptr(v), _ptr(csr_cols),
+                                       _ptr(csr_cnt), _ptr(out), B, Hq, Hkv, S, D, BLOCK, segment_size, *strides,
+                                       softmax_scale, _ptr(ws), _stream()),
                "pbs_sparse_attn_fwd")
     return out
 

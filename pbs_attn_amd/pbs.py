@@ -47,12 +47,12 @@ class PermutedKV:
     perm_vt: torch.Tensor       # (B, Hq, nb, D, 128): V blocks transposed [d][key]
     pooled_k: torch.Tensor      # (B, Hq, nb, D)
     seq_len: int
-    key_states: torch.Tensor = None   # the caller's K (B, Hkv or Hq, S, D), read in place for own-segment tiles
-    orig_vt: torch.Tensor = None      # (B, Hkv, nb, D, 128): V blocks in original order, transposed
+    key_states: torch.Tensor = None     # the caller's K and V (B, Hkv or Hq, S, D), read in place for own-segment tiles
+    value_states: torch.Tensor = None
 
     def attention(self, query_states, csr_cols, csr_cnt, segment_size, softmax_scale=None, out=None):
         """Sparse attention over this permutation (see ops.sparse_attn_fwd)."""
-        return ops.sparse_attn_fwd(query_states, self.perm_k, self.perm_vt, self.key_states, self.orig_vt,
+        return ops.sparse_attn_fwd(query_states, self.perm_k, self.perm_vt, self.key_states, self.value_states,
                                    csr_cols, csr_cnt, segment_size, softmax_scale, out)
 
     def permuted_keys(self):
@@ -84,10 +84,9 @@ def apply_permutation(query_states, key_states, value_states, block_size, segmen
             _mark("score")
         idx = ops.segment_argsort(scores, S, segment_size, block_size)
         _mark("sort")
-    perm_k, perm_vt, pooled_k, orig_vt = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode,
-                                                       want_orig_vt=True)
+    perm_k, perm_vt, pooled_k = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode)
     _mark("gather")
-    return PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, orig_vt)
+    return PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, value_states)
 
 
 def permuted_block_selection(query_states, perm: PermutedKV, block_size, segment_size, threshold=0.9, causal=True,
@@ -139,10 +138,10 @@ def _select_then_gather(query_states, key_states, value_states, block_size, segm
     _, _, cols, cnt = ops.select_blocks(P, threshold, idx, S, block_size, segment_size, force_select_first_block,
                                         want_masks=False, block_needed=needed, candidate_rule=1)
     _mark("select")
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode, want_orig_vt=True,
+    perm_k, perm_vt, _ = ops.gather_kv(key_states, value_states, idx, Hq, key_pool_mode,
                                                 block_needed=needed, want_pooled=False)
     _mark("gather")
-    perm = PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, orig_vt)
+    perm = PermutedKV(idx, perm_k, perm_vt, pooled_k, S, key_states, value_states)
     return perm, dict(block_attn_scores=P, csr_cols=cols, csr_cnt=cnt, block_needed=needed)
 
 

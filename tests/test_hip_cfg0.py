@@ -34,9 +34,9 @@ def test_cfg0_stages_bit_exact_on_the_oracle_scores(dev, cfg0):
     assert torch.equal(sel.cpu(), mid["block_mask"]), "block mask differs on identical block probabilities"
     assert torch.equal(fin.cpu(), mid["final_mask"])
     kd, vd = k.to(dev), v.to(dev)
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx, Hq)
     assert torch.equal(perm_k.cpu(), mid["perm_k"])
-    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, orig_vt, cols, cnt, 256).cpu()
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, vd, cols, cnt, 256).cpu()
     dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], mid["key_indices"], mid["final_mask"], 128)
     assert_attn_close(out, dense, MAX_ABS, MEAN_ABS, "HIP vs dense fp32 oracle on the oracle's mask")
     assert_attn_close(out, cfg0["ref"], MAX_ABS, MEAN_ABS, "HIP vs the oracle's naive path")

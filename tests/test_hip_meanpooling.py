@@ -35,8 +35,8 @@ def test_meanpooling_masks_bit_exact_and_output_vs_dense(dev, B, Hq, Hkv, S, thr
     # the selection on the ORACLE's block probabilities: masks must be bit-exact
     sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, ff)
     assert torch.equal(fin.cpu(), mid["block_mask"])
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
-    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128).cpu()
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx, Hq)
+    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, vd, cols, cnt, 128).cpu()
     dense = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128)
     assert_attn_close(out, dense, what="MeanPooling HIP vs dense fp32 on the oracle's mask")
     assert_attn_close(ref_out, dense, max_abs=2.5e-2, what="oracle naive vs dense fp32")
@@ -79,15 +79,15 @@ def test_meanpooling_with_an_optional_diagonal_block(dev, B, Hq, Hkv, S, thr, ff
     sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, ff, candidate_rule=2)
     assert torch.equal(sel.cpu(), mid["block_mask"])
     own = sel.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
-    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=own).cpu()
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx, Hq)
+    out = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, vd, cols, cnt, 128, own_block_needed=own).cpu()
     dense = O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128)
     assert_attn_close(out, dense, what="optional diagonal: HIP vs dense fp32 on the oracle's mask")
     assert_attn_close(ref_out, dense, max_abs=2.5e-2, what="oracle naive vs dense fp32")
     # with every flag set the entry point is the plain one
     ones = torch.ones_like(own)
-    a = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=ones)
-    b = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128)
+    a = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, vd, cols, cnt, 128, own_block_needed=ones)
+    b = ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, vd, cols, cnt, 128)
     assert torch.equal(a, b)
     # the whole mode from raw Q, K, V
     out2, got = MeanPooling_prefill(qd, kd, vd, 128, 1024, thr, True, ff, False, return_masks=True)
@@ -143,9 +143,9 @@ def test_query_blocks_that_select_nothing_give_zeros(dev, B, Hq, Hkv, S, thr):
     sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), float(thr), idx, S, 128, 128, False, candidate_rule=2)
     assert torch.equal(sel.cpu(), mid["block_mask"])
     own = sel.diagonal(dim1=-2, dim2=-1).to(torch.uint8).contiguous()
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx, Hq)
     out = torch.full_like(qd, float("nan"))
-    ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, orig_vt, cols, cnt, 128, own_block_needed=own, out=out)
+    ops.sparse_attn_fwd(qd, perm_k, perm_vt, kd, vd, cols, cnt, 128, own_block_needed=own, out=out)
     out = out.cpu()
     dense = torch.nan_to_num(O.dense_masked_attention_fp32(q, ke, ve, mid["key_indices"], mid["block_mask"], 128), nan=0.0)
     assert_attn_close(out, dense, what="rows without blocks: HIP vs dense fp32 (zeros where nothing is selected)")

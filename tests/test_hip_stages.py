@@ -215,10 +215,10 @@ def _run_attention_case(dev, B, Hq, Hkv, S, seg, thr, seed):
     idx_pad = torch.cat([idx, torch.arange(S, nb * 128).expand(B, Hq, -1)], -1).int().contiguous().to(dev)
     # same indices and same block probabilities as the oracle -> same masks (asserted), then attention
     kd, vd = k.to(dev), v.to(dev)
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx_pad, Hq, want_orig_vt=True)
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx_pad, Hq)
     sel, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), thr, idx_pad, S, 128, seg, True)
     assert torch.equal(fin.cpu(), mid["final_mask"])
-    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, orig_vt, cols, cnt, seg).cpu()
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, vd, cols, cnt, seg).cpu()
     dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], idx, mid["final_mask"], 128)
     assert_attn_close(out, out_ref, what="HIP vs oracle naive path")
     assert_attn_close(out, dense, what="HIP vs dense fp32 oracle")
@@ -238,7 +238,7 @@ def test_sparse_attention_strided_query(dev):
     qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
     perm = P.apply_permutation(qd, kd, vd, 128, 256)
     sel = P.permuted_block_selection(qd, perm, 128, 256, 0.9)
-    args = (perm.perm_k, perm.perm_vt, perm.key_states, perm.orig_vt, sel["csr_cols"], sel["csr_cnt"], 256)
+    args = (perm.perm_k, perm.perm_vt, perm.key_states, perm.value_states, sel["csr_cols"], sel["csr_cnt"], 256)
     q_strided = qd.transpose(1, 2).contiguous().transpose(1, 2)
     assert not q_strided.is_contiguous()
     out_c = ops.sparse_attn_fwd(qd, *args)
@@ -260,10 +260,10 @@ def test_reference_naive_path_is_the_outlier_on_short_rows(dev):
     ref, mid = O.permuted_block_sparse_attn_fwd(q, ke, ve, 128, 256, 0.9, return_intermediates=True)
     idx_pad = mid["key_indices"].int().contiguous().to(dev)
     kd, vd = k.to(dev), v.to(dev)
-    perm_k, perm_vt, _, orig_vt = ops.gather_kv(kd, vd, idx_pad, 4, want_orig_vt=True)
+    perm_k, perm_vt, _ = ops.gather_kv(kd, vd, idx_pad, 4)
     _, fin, cols, cnt = ops.select_blocks(mid["block_attn_scores"].to(dev), 0.9, idx_pad, 768, 128, 256, True)
     assert torch.equal(fin.cpu(), mid["final_mask"])
-    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, orig_vt, cols, cnt, 256).cpu()
+    out = ops.sparse_attn_fwd(q.to(dev), perm_k, perm_vt, kd, vd, cols, cnt, 256).cpu()
     dense = O.dense_masked_attention_fp32(q, mid["perm_k"], mid["perm_v"], mid["key_indices"], mid["final_mask"], 128)
     hip_err = (out.float() - dense).abs()
     naive_err = (ref.float() - dense).abs()
@@ -583,16 +583,15 @@ def test_selection_marks_the_visited_blocks_and_the_filtered_gather_moves_exactl
     assert torch.equal(needed, want)
     if isinstance(thr, float):
         assert 0 < int(needed.sum()) < needed.numel()        # the cases are meant to filter something
-    full_k, full_vt, _, full_ovt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True)
-    part_k, part_vt, none_pooled, part_ovt = ops.gather_kv(kd, vd, idx, Hq, want_orig_vt=True, block_needed=needed,
-                                                            want_pooled=False)
-    assert none_pooled is None and torch.equal(part_ovt, full_ovt)
+    full_k, full_vt, _ = ops.gather_kv(kd, vd, idx, Hq)
+    part_k, part_vt, none_pooled = ops.gather_kv(kd, vd, idx, Hq, block_needed=needed, want_pooled=False)
+    assert none_pooled is None
     m = needed.bool()
     assert torch.equal(part_k.view(B, Hq, nb, 128, 128)[m], full_k.view(B, Hq, nb, 128, 128)[m])
     assert torch.equal(part_vt[m], full_vt[m])
     # and the attention over the partly gathered tiles is the attention over the full ones, bit for bit
-    out_full = ops.sparse_attn_fwd(qd, full_k, full_vt, kd, full_ovt, cols, cnt, seg)
-    out_part = ops.sparse_attn_fwd(qd, part_k, part_vt, kd, part_ovt, cols, cnt, seg)
+    out_full = ops.sparse_attn_fwd(qd, full_k, full_vt, kd, vd, cols, cnt, seg)
+    out_part = ops.sparse_attn_fwd(qd, part_k, part_vt, kd, vd, cols, cnt, seg)
     assert torch.equal(out_full, out_part)
 
 
@@ -609,7 +608,7 @@ def test_filtered_gather_leaves_unneeded_tiles_alone(dev):
     pk = torch.full_like(lib_k, 7.0)
     pvt = torch.full_like(lib_vt, 7.0)
     lib = L.load()
-    L.check(lib.pbs_gather_kv(_ptr(kd), _ptr(vd), _ptr(idx), _ptr(pk), _ptr(pvt), None, None, 1, 2, 2, 1024, 128, 128,
+    L.check(lib.pbs_gather_kv(_ptr(kd), _ptr(vd), _ptr(idx), _ptr(pk), _ptr(pvt), None, 1, 2, 2, 1024, 128, 128,
                               kd.stride(0), kd.stride(1), kd.stride(2), vd.stride(0), vd.stride(1), vd.stride(2), 0,
                               _ptr(needed), _stream()), "pbs_gather_kv")
     torch.cuda.synchronize()
