@@ -47,6 +47,7 @@
 #include "pbs_attn_tile.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <atomic>
+#include <type_traits>
 
 namespace {
 
@@ -143,10 +144,11 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
       int n = total;
       if (own_needed[(int64_t)bh * nb + qb0]) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG | (1u << 14));
       if (second && own_needed[(int64_t)bh * nb + qb1]) out[1 + n++] = (uint16_t)(qb1 | ENT_ORIG | (2u << 14));
-      // a pair that visits nothing still gets one tile (its own block, used by neither query block): the attention
-      // kernel's item protocol -- first tile in flight, claim and hand-over of the next item -- needs no empty case,
-      // and a query block that used no tile writes zeros
-      if (n == 0) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG);
+      // every list ends with an own-segment entry: a pair with neither own block listed gets the first one's, used by
+      // neither query block.  The attention kernel's item protocol -- first tile in flight, claim and hand-over of the
+      // next item at the last tiles -- then needs no empty case and none where a permuted tile ends the item; a query
+      // block that used no tile writes zeros
+      if (n == total) out[1 + n++] = (uint16_t)(qb0 | ENT_ORIG);
       out[0] = (uint16_t)n;
     }
     return;
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     uint32_t k_ss, v_ss;
     int S;
   };
-  auto head_base = [&](ArgsPtr ap, int bh_e) {
+  auto head_base = [&](ArgsPtr ap, int bh_e) __attribute__((always_inline)) {
     HeadBase hb;
     const int Hq_e = ap->Hq, Hkv_e = ap->Hkv, nb_e = ap->nb;
     const int b_e = bh_e / Hq_e, kvh = (bh_e % Hq_e) / (Hq_e / Hkv_e);
@@ -253,7 +255,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     return hb;
   };
   // copy of one visit-list entry's K and V^T tiles into the buffers at LDS byte offset `buf`
-  auto stage_entry = [&](const HeadBase& hb, uint32_t e, uint32_t buf, int lane, uint32_t lane_off) {
+  auto stage_entry = [&](const HeadBase& hb, uint32_t e, uint32_t buf, int lane, uint32_t lane_off) __attribute__((always_inline)) {
     const int kb_e = (int)(e & ENT_KB);
     if (PBS_UNLIKELY(e & ENT_ORIG)) {
       // the lane id is formed afresh: offsets derived from the item's one are loop invariants that get hoisted out of
@@ -265,7 +267,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       stage_tile_async(hb.pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
     }
   };
-  auto list_row = [&](ArgsPtr ap, int item) {
+  auto list_row = [&](ArgsPtr ap, int item) __attribute__((always_inline)) {
     const int bh_i = item / npair, pair_i = npair - 1 - item % npair;
     return ap->plist + ((int64_t)bh_i * npair + pair_i) * ap->cap;
   };
@@ -331,10 +333,10 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
     // tile), published and its list and queries requested one tile later, its first tile requested at the last
     // tile.  Items of fewer than three tiles finish these steps after their loop.
     const int claim_it = careful_only ? -8 : max(n_tiles - 3, 0);
-    auto publish_and_fetch = [&]() {   // between the wait for this thread's loads and the barrier ...
+    auto publish_and_fetch = [&]() __attribute__((always_inline)) {   // between the wait for this thread's loads and the barrier ...
       if (wave == 0 && lane_id_here() == 0) misc[4] = q_begin + claim;
     };
-    auto adopt_next = [&]() {          // ... and after the barrier
+    auto adopt_next = [&]() __attribute__((always_inline)) {          // ... and after the barrier
       nxt = ticket_item(q_begin, q_end, __builtin_amdgcn_readfirstlane(misc[4]), PBS_ARGS()->interleave, npair);
       has_nxt = nxt < q_end;
       if (has_nxt) {
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
             for (int r = 0; r < 4; ++r) o[dt][qg][r] = zero;
       }
       float m_ref[2] = {-INFINITY, -INFINITY};   // reference maxima of queries i16 and 16 + i16, identical in the four lanes i16 + 16 g
-      float l_part[2] = {0.f, 0.f};              // row sums over this lane's quarter of the keys
+      float l_row[2] = {0.f, 0.f};               // row sums of queries i16 and 16 + i16, identical in the four lanes too
       bool first = true, poisoned = false;
       bool all_seen = false;     // every query of this wave has a finite reference maximum (wave-uniform)
 
@@ -387,7 +389,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1]), par, lane, lane_off);
       }
       uint32_t bufx = par;
-      auto next_buffers = [&]() {
+      auto next_buffers = [&]() __attribute__((always_inline)) {
         bufx ^= 0x8000u;
 #pragma unroll
         for (int n = 0; n < 4; ++n) {
@@ -397,19 +399,25 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       };
       // what every tile starts with: wait for its copies, hand over the buffers of the tile before, and request the
       // copies of the tile after it (or, at the last tile, of the next item's first tile)
-      auto tile_head = [&](int it) {
+      // `may_be_last`: the item's last tile is an own-segment tile (merge_pair_lists_kernel ends every list with one),
+      // so the loop over the permuted tiles always has a next entry to request and carries no code for the next item's
+      // first tile
+      auto tile_head = [&](int it, auto may_be_last) __attribute__((always_inline)) {
         __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0): this thread's share of tile `it` (and of the next list) has landed
         if (PBS_UNLIKELY(it == claim_it + 1)) publish_and_fetch();
         __syncthreads();                      // every share has; every wave is done with tile it - 1
         if (PBS_UNLIKELY(it == claim_it + 1)) adopt_next();
         if (PBS_UNLIKELY(it == claim_it) && wave == 0 && lane_id_here() == 0) claim = atomicAdd(PBS_ARGS()->queue + vic, 1);
-        if (PBS_LIKELY(it + 1 < n_tiles)) stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
+        if (!decltype(may_be_last)::value || PBS_LIKELY(it + 1 < n_tiles))
+          stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
         else if (has_nxt && (careful_only || n_tiles >= 3))   // shorter items: after the loop, once the list has landed
           stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx ^ 0x8000u, lane, lane_off);
       };
+      constexpr std::integral_constant<bool, true> any_tile{};
+      constexpr std::integral_constant<bool, false> not_the_last{};
       // first tile of a row, every key visible: the exact maximum over its first 32 keys is a good enough reference
       // to start the pipelined path (later keys move it up lazily)
-      auto first_reference = [&]() {
+      auto first_reference = [&]() __attribute__((always_inline)) {
         first = false;
         float mx[2] = {-INFINITY, -INFINITY};
 #pragma unroll
@@ -432,7 +440,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       };
       // careful tile: classic online softmax, one 32-key sub-tile at a time.  The redo pass, and a diagonal tile
       // while some query has not seen a single key yet (its reference maximum is still -inf)
-      auto careful_tile = [&](uint32_t ent, bool masked) {
+      auto careful_tile = [&](uint32_t ent, bool masked) __attribute__((always_inline)) {
         first = false;
 #pragma nounroll
         for (int ks = 0; ks < 4; ++ks) {   // a real loop: the rare path stays small, in code and in registers
@@ -477,7 +485,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
               rs += pe;
               pf[qg][e] = (__bf16)pe;
             }
-            l_part[qg] = l_part[qg] * alpha[qg] + rs;
+            l_row[qg] = l_row[qg] * alpha[qg] + sum_over_lane_groups(rs);
           }
           if (__any(alpha[0] != 1.0f || alpha[1] != 1.0f)) {
 #pragma unroll
@@ -498,37 +506,48 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         }
         all_seen = !__any(m_ref[0] == -INFINITY || m_ref[1] == -INFINITY);
       };
-      // The merged list holds the permuted tiles of earlier segments first, then the tiles of the own segments.  Each
-      // kind has a loop of its own, and so has the redo pass: a loop whose body updates the 64 accumulator registers
-      // on one path only keeps them in place, where several alternative tile bodies in one loop cost a copy of all of
-      // them per tile.
+      // The merged list holds the permuted tiles of earlier segments first, then the tiles of the own segments in
+      // ascending order: for a query block those before its own block, its own (diagonal) block, and -- for the first
+      // block of a pair -- the second block's, which it skips.  Each kind has a loop of its own, and so has the redo
+      // pass: a loop whose body updates the 64 accumulator registers on one path only keeps them in place, where
+      // alternative tile bodies inside one loop cost a copy of all of them per tile (and the registers for it).
       int it = 0;
+      auto entry = [&](int i) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + i]); };
       if (PBS_UNLIKELY(careful_only)) {
         for (; it < n_tiles; ++it, next_buffers()) {
-          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
-          tile_head(it);
+          const uint32_t ent = entry(it);
+          tile_head(it, any_tile);
           if (!(ent & use_bit) || !qb_valid) continue;
           careful_tile(ent, (ent & ENT_ORIG) && (int)(ent & ENT_KB) == qb);
         }
       } else {
-        for (; it < n_tiles; ++it, next_buffers()) {
-          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
+        for (; it < n_tiles; ++it, next_buffers()) {          // permuted tiles
+          const uint32_t ent = entry(it);
           if (PBS_UNLIKELY(ent & ENT_ORIG)) break;
-          tile_head(it);
+          tile_head(it, not_the_last);
           if (PBS_UNLIKELY(!(ent & use_bit) || !qb_valid)) continue;
           if (PBS_UNLIKELY(first)) first_reference();
-          fast_tile<false, PREFETCH_SLOTS, false>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+          fast_tile<false, PREFETCH_SLOTS, false>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
         }
-        for (; it < n_tiles; ++it, next_buffers()) {
-          const uint32_t ent = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + it]);
-          tile_head(it);
+        for (; it < n_tiles; ++it, next_buffers()) {          // own-segment tiles before the diagonal: every key visible
+          const uint32_t ent = entry(it);
+          if ((int)(ent & ENT_KB) >= qb) break;
+          tile_head(it, any_tile);
           if (!(ent & use_bit) || !qb_valid) continue;
-          const bool masked = (int)(ent & ENT_KB) == qb;   // the diagonal block; other own-segment blocks lie before it
-          if (first && !masked) first_reference();
-          if (first || (masked && !all_seen)) careful_tile(ent, masked);
-          else if (masked) fast_tile<true, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
-          else fast_tile<false, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_part, poisoned, wq);
+          if (first) first_reference();
+          fast_tile<false, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
         }
+        if (it < n_tiles && (int)(entry(it) & ENT_KB) == qb) {   // the diagonal tile
+          const uint32_t ent = entry(it);
+          tile_head(it, any_tile);
+          if ((ent & use_bit) && qb_valid) {
+            if (first || !all_seen) careful_tile(ent, true);
+            else fast_tile<true, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
+          }
+          ++it;
+          next_buffers();
+        }
+        for (; it < n_tiles; ++it, next_buffers()) tile_head(it, any_tile);   // tiles of the pair's other block only
       }
       if (!careful_only && n_tiles < 3) {
         if (n_tiles < 2) {
@@ -557,7 +576,7 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       float inv[2];
 #pragma unroll
       for (int qg = 0; qg < 2; ++qg) {
-        const float l_all = sum_over_lane_groups(l_part[qg]);
+        const float l_all = l_row[qg];
         inv[qg] = l_all == 0.f ? 0.f : 1.0f / l_all;
       }
       // lane-dependent addresses of the epilogue come from a fresh opaque lane id: derived from the item's one

@@ -208,7 +208,7 @@ __device__ __forceinline__ float sum_over_lane_groups(float v) {
 template <bool MASKED, int PF, bool V_ROWS>
 __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2][4], const uint32_t (&ka)[4],
                                           const uint32_t (&va)[4], float c_log2, float (&m_ref)[2],
-                                          float (&l_part)[2], bool& poisoned, int wq) {
+                                          float (&l_row)[2], bool& poisoned, int wq) {
   // query-in-block minus the lane group's key offset; made opaque per call: the mask compares of a
   // diagonal tile depend only on the lane, and hoisted out of the tile loop they would each pin a 64-bit
   // scalar mask
@@ -220,7 +220,14 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
   const float negm[2] = {-m_ref[0], -m_ref[1]};
   uint32_t vr = 0;
   if (V_ROWS) vr = vrow_lane_addr(LDS_V0 + (va[0] & 0x8000u), lane_id_here());   // va[] carries the buffer switch in bit 15
-  float rsum[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  // row sums: one more matrix instruction per sub-tile and column group, ones x P, whose every output row is the sum
+  // over the sub-tile's 32 keys of the probabilities as the P.V product sees them (rounded to bf16).  Summing them
+  // with vector adds instead costs 64 vector instructions per tile, and the vector unit is as busy as the matrix
+  // unit here.
+  f32x4 lsum[2];
+  u32x4 one_bits = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+  asm volatile("" : "+v"(one_bits));
+  const bf16x8 ones = __builtin_bit_cast(bf16x8, one_bits);
   f32x4 sacc[2][2][2];     // [sub-tile parity][T][qg]
   bf16x8 pbuf[2][2];       // [sub-tile parity][qg]
   constexpr int R = PF + 1;
@@ -255,6 +262,10 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
     if (step >= 2) {
 #pragma unroll
       for (int qg = 0; qg < 2; ++qg) o[t][qg] = PBS_MFMA(frv[n % R], pbuf[step & 1][qg], o[t][qg]);
+      if (t == 1 || t == 5) {
+        const int qg = t >> 2;
+        lsum[qg] = PBS_MFMA(ones, pbuf[step & 1][qg], step == 2 ? (f32x4){0} : lsum[qg]);
+      }
     }
     if (step >= 1 && step <= 4) {
       const int sb = (step - 1) & 1, qg = t >> 2, T = (t >> 1) & 1, c0 = 2 * (t & 1);
@@ -267,16 +278,14 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
       }
       const float e0 = __builtin_amdgcn_exp2f(__builtin_fmaf(x0, c_log2, negm[qg]));
       const float e1 = __builtin_amdgcn_exp2f(__builtin_fmaf(x1, c_log2, negm[qg]));
-      rsum[qg][0] += e0;
-      rsum[qg][1] += e1;
       pbuf[sb][qg][4 * T + c0] = (__bf16)e0;
       pbuf[sb][qg][4 * T + c0 + 1] = (__bf16)e1;
     }
     __builtin_amdgcn_sched_barrier(0);
   }
-  const float rs[2] = {rsum[0][0] + rsum[0][1], rsum[1][0] + rsum[1][1]};
-  l_part[0] += rs[0];
-  l_part[1] += rs[1];
+  const float rs[2] = {lsum[0][0], lsum[1][0]};   // the whole row of this tile, the same in the four lanes of a query
+  l_row[0] += rs[0];
+  l_row[1] += rs[1];
   // lazy reference maximum without tracking maxima: a row sum of this tile above 2^14 says some
   // exponential was large; any reference >= the old one is valid, so move it up by log2(sum)
   if (PBS_UNLIKELY(__any(rs[0] > 16384.0f || rs[1] > 16384.0f))) {
@@ -287,7 +296,7 @@ __device__ __forceinline__ void fast_tile(f32x4 (&o)[8][2], const bf16x8 (&qf)[2
       const float m_new = (big > 16384.0f) ? m_ref[qg] + __builtin_amdgcn_logf(big) : m_ref[qg];
       const float alpha = __builtin_amdgcn_exp2f(m_ref[qg] - m_new);
       m_ref[qg] = m_new;
-      l_part[qg] *= alpha;
+      l_row[qg] *= alpha;
 #pragma unroll
       for (int dt = 0; dt < 8; ++dt)
 #pragma unroll
