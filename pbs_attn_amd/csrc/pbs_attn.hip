@@ -263,8 +263,17 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       stage_krows_async(hb.korig + (int64_t)kb_e * BS * hb.k_ss, hb.k_ss, hb.S - kb_e * BS, buf, wave, lane_id_here());
       stage_vrows_async(hb.vorig + (int64_t)kb_e * BS * hb.v_ss, hb.v_ss, hb.S - kb_e * BS, LDS_V0 + buf, wave, lane_id_here());
     } else {
-      stage_tile_async(hb.pk + (int64_t)kb_e * BS * D, buf, wave, lane_off ^ k_copy_xor(wave));
-      stage_tile_async(hb.pvt + (int64_t)kb_e * BS * D, LDS_V0 + buf, wave, lane_off);
+      // the first wave of every SIMD issues its own share and that of the SIMD's second wave (rows 16 further: the
+      // same chunk, 4096 bytes on), which goes straight on to the matrix instructions of the current tile: the copy
+      // instructions of a tile then queue behind the barrier in four waves instead of eight
+      if (wave < 4) {
+        const uint16_t* ks = hb.pk + (int64_t)kb_e * BS * D;
+        const uint16_t* vs = hb.pvt + (int64_t)kb_e * BS * D;
+        stage_tile_async(ks, buf, wave, lane_off ^ k_copy_xor(wave));
+        stage_tile_async(ks, buf, wave + 4, (lane_off + 4096u) ^ k_copy_xor(wave + 4));
+        stage_tile_async(vs, LDS_V0 + buf, wave, lane_off);
+        stage_tile_async(vs, LDS_V0 + buf, wave + 4, lane_off + 4096u);
+      }
     }
   };
   auto list_row = [&](ArgsPtr ap, int item) __attribute__((always_inline)) {

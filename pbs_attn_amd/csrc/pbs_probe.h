@@ -18,7 +18,8 @@ double pbs_mfma_probe_flop(int iters);
  * workgroups of 8 waves each run `iters` unmasked 128-key tiles for their 256 queries (2 x 128 x 128 block pairs
  * per workgroup and tile, 8.389 MFLOP each) out of LDS, with the kernel's barrier per tile and, if `with_copies`,
  * its asynchronous copies of the next tile (64 KB from a ring of `n_src_tiles` >= 2 K / V^T tile pairs of 65536
- * bytes each at `tiles`, whose first 32 KB also serve as the queries) -- no visit lists, no write-out.  `sink`
+ * bytes each at `tiles`, whose first 32 KB also serve as the queries; the workgroups of an XCD copy the same tile at
+ * the same step, as the kernel's share a head's stream in their L2) -- no visit lists, no write-out.  `sink`
  * takes 256 * 512 floats; `clocks` receives workgroup 0's shader-clock ticks and 100 MHz ticks.  `with_copies`
  * bit 1 handles the tiles as a tile of the query block's own segment is handled: K and V copied row by row, the V
  * fragments formed by transposing reads.  Time the launch

@@ -113,13 +113,19 @@ __global__ __launch_bounds__(512, 2) void tile_probe_kernel(const uint16_t* __re
     __builtin_amdgcn_s_waitcnt(0x0f70);
     __syncthreads();
     if (with_copies) {
-      const uint16_t* src = tiles + (size_t)((it * 7 + (int)blockIdx.x / 8) % n_src) * (2 * BS * D);
+      // the 32 workgroups of an XCD (blockIdx % 8) copy the same tile at the same step, as the kernel's workgroups
+      // of an XCD walk one head's K / V stream together and share it in that XCD's L2
+      const uint16_t* src = tiles + (size_t)((it * 7 + (int)(blockIdx.x & 7) * 29) % n_src) * (2 * BS * D);
       if (V_ROWS) {
         stage_krows_async(src, D, BS, bufx ^ 0x8000u, wave, lane_id_here());
         stage_vrows_async(src + BS * D, D, BS, LDS_V0 + (bufx ^ 0x8000u), wave, lane_id_here());
       } else {
-        stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off ^ k_copy_xor(wave));
-        stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+        if (wave < 4) {   // as the kernel does: the first wave of every SIMD issues the second wave's share too
+          stage_tile_async(src, bufx ^ 0x8000u, wave, lane_off ^ k_copy_xor(wave));
+          stage_tile_async(src, bufx ^ 0x8000u, wave + 4, (lane_off + 4096u) ^ k_copy_xor(wave + 4));
+          stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave, lane_off);
+          stage_tile_async(src + BS * D, LDS_V0 + (bufx ^ 0x8000u), wave + 4, lane_off + 4096u);
+        }
       }
     }
     uint32_t ka[4], va[4];
