@@ -43,7 +43,7 @@ int pbs_score_keys(const void* q, const void* k, float* scores, int B, int Hq, i
  * statistics live in a library-owned device array of PBS_SCORE_KEYS_STATIC_SCRATCH_BYTES per GPU (held
  * until the process ends); shapes whose pbs_score_keys_workspace_bytes exceeds it are rejected with an
  * argument error (-1).  The device address of the array is looked up on the first call on each device
- * (-2 if that fails).  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
+ * (-2 if that fails): make that first call outside any stream capture.  All calls on one GPU share the array: calls that overlap on one GPU (two streams,
  * two threads) race; calls on one stream are ordered and safe.  Same arguments, results and error
  * behaviour as pbs_score_keys otherwise. */
 #define PBS_SCORE_KEYS_STATIC_SCRATCH_BYTES ((size_t)8 << 20)
