@@ -12,6 +12,7 @@
 // Rows of up to 1024 blocks take the wave-level variant further down (one wave per row,
 // the row in registers).
 #include "pbs_common.h"
+#include <utility>
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <float.h>
 
@@ -253,14 +254,13 @@ __device__ __forceinline__ void wave_bitonic_sort_u32(uint32_t (&k)[NPL], int la
   }
 }
 
+// one wave decides row `rq` ((row, qb - qb_lo) flattened) of the group of rows [qb_lo, qb_hi) x all heads
 template <int NPL>
-__global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, int total_rows) {
-  extern __shared__ uint8_t smem_w[];
+__device__ __forceinline__ void select_row_by_wave(const SelectArgs& a, int64_t rq, int total_rows, uint8_t* smem_w) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int nb = a.nb;
   const int nb_pad = (nb + 15) & ~15;
   uint8_t* flag = smem_w + wave * nb_pad;
-  const int64_t rq = (int64_t)blockIdx.x * 4 + wave;   // (row, qb - qb_lo) flattened
   if (rq >= total_rows) return;
   const int nqb = a.qb_hi - a.qb_lo;
   const int row = (int)(rq / nqb), qb = a.qb_lo + (int)(rq % nqb);
@@ -468,6 +468,37 @@ __global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, i
   if (lane == 0) a.csr_cnt[(int64_t)row * nb + qb] = base;
 }
 
+template <int NPL>
+__global__ __launch_bounds__(256) void select_blocks_wave_kernel(SelectArgs a, int total_rows) {
+  extern __shared__ uint8_t smem_w[];
+  select_row_by_wave<NPL>(a, (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6), total_rows, smem_w);
+}
+
+// Up to five groups of rows of like length (see pbs_select_blocks) in ONE launch, the longest rows first: as launches
+// of their own the groups run one after the other and each ends with a tail of idle CUs.
+struct SelectGroups {
+  int n;
+  int npl[5], qb_lo[5], qb_hi[5];
+  int wg_end[5];   // workgroups of groups 0 .. g
+};
+__global__ __launch_bounds__(256) void select_blocks_groups_kernel(SelectArgs a, SelectGroups gr, int rows) {
+  extern __shared__ uint8_t smem_w[];
+  int g = 0;
+  while (g + 1 < gr.n && (int)blockIdx.x >= gr.wg_end[g]) ++g;
+  const int wg0 = g == 0 ? 0 : gr.wg_end[g - 1];
+  a.qb_lo = gr.qb_lo[g];
+  a.qb_hi = gr.qb_hi[g];
+  const int total = rows * (a.qb_hi - a.qb_lo);
+  const int64_t rq = (int64_t)((int)blockIdx.x - wg0) * 4 + (threadIdx.x >> 6);
+  switch (gr.npl[g]) {
+    case 1: select_row_by_wave<1>(a, rq, total, smem_w); break;
+    case 2: select_row_by_wave<2>(a, rq, total, smem_w); break;
+    case 4: select_row_by_wave<4>(a, rq, total, smem_w); break;
+    case 8: select_row_by_wave<8>(a, rq, total, smem_w); break;
+    default: select_row_by_wave<16>(a, rq, total, smem_w); break;
+  }
+}
+
 // Visit lists from a given block mask: one wave per (row, query block), the set bits of strictly earlier segments
 // compacted in ascending order; own_missing counts the blocks of the query block's own segment the mask leaves out
 // (in permuted order any of them can hold keys the query may see).
@@ -558,6 +589,8 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
     if (candidate_rule == 0 || threshold_is_int_one) {
       launch(threshold_is_int_one || nb <= 64 ? 1 : nb <= 128 ? 2 : nb <= 256 ? 4 : nb <= 512 ? 8 : 16, 0, nb);
     } else {
+      SelectGroups gr;
+      gr.n = 0;
       int qb_lo = 0;
       for (int npl = 1; npl <= 16 && qb_lo < nb; npl *= 2) {
         // query blocks whose candidate count fits 64 * npl sorted entries
@@ -565,9 +598,26 @@ extern "C" int pbs_select_blocks(const float* block_attn_scores, const float* th
         int64_t hi = candidate_rule == 1 ? (lim / bps + 1) * (int64_t)bps : lim;
         if (npl == 16 || hi > nb) hi = nb;
         if (hi > qb_lo) {
-          launch(npl, qb_lo, (int)hi);
+          gr.npl[gr.n] = npl; gr.qb_lo[gr.n] = qb_lo; gr.qb_hi[gr.n] = (int)hi;
+          ++gr.n;
           qb_lo = (int)hi;
         }
+      }
+      if (gr.n == 1) {
+        launch(gr.npl[0], gr.qb_lo[0], gr.qb_hi[0]);
+      } else {
+        // longest rows first
+        for (int x = 0; x < gr.n / 2; ++x) {
+          std::swap(gr.npl[x], gr.npl[gr.n - 1 - x]);
+          std::swap(gr.qb_lo[x], gr.qb_lo[gr.n - 1 - x]);
+          std::swap(gr.qb_hi[x], gr.qb_hi[gr.n - 1 - x]);
+        }
+        int wgs = 0;
+        for (int x = 0; x < gr.n; ++x) {
+          wgs += (rows * (gr.qb_hi[x] - gr.qb_lo[x]) + 3) / 4;
+          gr.wg_end[x] = wgs;
+        }
+        hipLaunchKernelGGL(select_blocks_groups_kernel, dim3((unsigned)wgs), dim3(256), lds_w, st, a, gr, rows);
       }
     }
     return pbs_check_launch("pbs_select_blocks");
