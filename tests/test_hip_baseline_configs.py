@@ -64,7 +64,18 @@ def _check_selection(Pm, chosen, final, cnt, cols, needed, first_col, thr, nb, b
     assert torch.equal(needed.bool(), visited.any(-2))      # marked for the gather <=> on some query block's list
 
 
-def _check_config(dev, name, sample_blocks, oracle_heads, **override):
+def _assert_close_with_large_values(out, ref, what):
+    """max-abs 2e-2 / mean-abs 2e-3, except that an element whose reference value is large may be off by 1.5 units in
+    the last place of bf16 (the rule of the random-configuration sweep: the strong_heavy inputs produce outputs beyond
+    +-4, where one bf16 step is 0.031 and the rounding of the output alone can take 0.016)."""
+    diff = (out.float() - ref.float()).abs()
+    assert torch.isfinite(out.float()).all(), what
+    ulp = torch.exp2(torch.floor(torch.log2(ref.abs().clamp_min(1e-30))) - 7)
+    assert (diff <= torch.maximum(torch.full_like(diff, 2e-2), 1.5 * ulp)).all(), (what, diff.max().item())
+    assert diff.mean().item() <= 2e-3, (what, diff.mean().item())
+
+
+def _check_config(dev, name, sample_blocks, oracle_heads, large_outputs=False, **override):
     cfg, q, k, v = make_workload(name, device=dev, **override)
     B, Hq, Hkv, S, seg, thr = cfg["B"], cfg["Hq"], cfg["Hkv"], cfg["S"], cfg["segment"], cfg["threshold"]
     nb, bps, G = S // 128, seg // 128, Hq // Hkv
@@ -109,7 +120,11 @@ def _check_config(dev, name, sample_blocks, oracle_heads, **override):
             logits = q[:, hs, rows].float() @ kf.transpose(-1, -2) / math.sqrt(128)
             allowed = torch.gather(final[:, hs, qb], -1, key_block[:, hs]).unsqueeze(2) & (pos.view(1, 1, 1, S) <= pos[rows].view(1, 1, -1, 1))
             ref = torch.softmax(logits.masked_fill(~allowed, float("-inf")), -1) @ vf
-            assert_attn_close(one[:, hs, rows], ref, what=f"{name}: query block {qb}, heads {h0}..{h0 + G - 1}")
+            what = f"{name}: query block {qb}, heads {h0}..{h0 + G - 1}"
+            if large_outputs:
+                _assert_close_with_large_values(one[:, hs, rows], ref, what)
+            else:
+                assert_attn_close(one[:, hs, rows], ref, what=what)
             worst = max(worst, (one[:, hs, rows].float() - ref).abs().max().item())
     print(f"{name}: {len(sample_blocks)} query blocks x {B * Hq} heads against dense fp32 on the path's mask: max-abs {worst:.2e}")
 
@@ -147,3 +162,9 @@ def test_cfg1_full_layer_threshold_09_segment_1024(dev):
 
 def test_cfg1_full_layer_segment_256(dev):
     _check_config(dev, "cfg1", sample_blocks=(1, 200), oracle_heads=[(0, 30)])
+
+
+def test_cfg2_shape_in_the_sparse_regime(dev):
+    # the supplementary strong_heavy input at cfg2's shape and parameters: 1.5 % of the causal blocks, 2 % of the
+    # permuted key blocks gathered, rows decided without a sort, items of 8 tiles
+    _check_config(dev, "cfg2", sample_blocks=(8, 517, 1023), oracle_heads=[(0, 3)], large_outputs=True, kind="strong_heavy")
