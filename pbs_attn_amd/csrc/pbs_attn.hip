@@ -25,15 +25,16 @@
 // Data layout
 //   K tile: 128 keys x 128 d row-major; permuted V tile: stored TRANSPOSED in HBM by the gather kernel,
 //   128 d x 128 keys; V tile of an own segment: 128 keys x 128 d as in the caller's tensor, its MFMA fragments
-//   read with the transposing LDS read.  Both sit in LDS as 128 rows x 16 chunks of 16 bytes with chunk index XOR
-//   (row & 15): v_mfma fragment reads (row = lane % 32, 16 bytes) are bank-conflict free.
-// Math (transposed formulation, v_mfma_f32_32x32x16_bf16)
+//   read with the transposing LDS read.  K and V^T tiles sit in LDS as 128 rows x 16 chunks of 16 bytes with the
+//   chunk index XORed with a hash of the row (pbs_attn_tile.h), so that fragment reads are bank-conflict free.
+// Math (transposed formulation, v_mfma_f32_16x16x32_bf16)
 //     S^T = K Q^T   (rows = keys, columns = queries)      O^T += V^T P^T   (rows = d, columns = queries)
-//   Every lane owns ONE query column, so softmax statistics are per-lane values, and the S^T
-//   accumulator registers are, after conversion to bf16, exactly the B operand of the second
-//   product (the key rows of each 32-row MFMA tile are fed in the order that makes this so).
-//   Softmax runs in the exp2 domain in fp32; P is rounded to bf16 before P.V and the row sum uses
-//   the unrounded values; the output is normalised once at the end.
+//   Every lane owns query columns (one per column group of 16 queries), so the softmax reference values are
+//   per-lane, and the S^T accumulator registers are, after conversion to bf16, exactly the B operand of the
+//   second product (the key rows of each 16-row MFMA tile are fed in the order that makes this so).
+//   Softmax runs in the exp2 domain in fp32; P is rounded to bf16 before P.V, and a pipelined tile takes its row
+//   sums from one more matrix product, ones x P, i.e. of the rounded values; the output is normalised once at
+//   the end.
 // Tile kinds
 //   * fast tiles: a software pipeline over the four 32-key sub-tiles -- S of sub-tile k+1, exponentials
 //     of sub-tile k and P.V of sub-tile k-1 are issued interleaved, LDS fragments are read two slots
@@ -42,8 +43,10 @@
 //     overflow marks the row and the whole workgroup redoes it without speculation.  The first tile of a
 //     row takes its reference from the exact maximum over its first 32 keys.  The diagonal tile runs the
 //     same pipeline and zeroes the exponentials of keys after the query (key-in-tile > query-in-block).
-//   * careful tiles (a row whose first tile is the diagonal one, and the redo pass): all of S first,
-//     exact running maximum, classic online softmax.
+//   * careful tiles (a row whose first tile is the diagonal one, and the redo pass): one 32-key sub-tile at a
+//     time, exact running maximum, classic online softmax.
+//   An item's tiles come in the order permuted tiles, own-segment tiles before the diagonal, diagonal tile, and
+//   each kind has a loop of its own (see the loops): one tile body per loop keeps the accumulators in place.
 #include "pbs_attn_tile.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 #include <atomic>
