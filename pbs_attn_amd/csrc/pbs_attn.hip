@@ -411,6 +411,9 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       };
       // what every tile starts with: wait for its copies, hand over the buffers of the tile before, and request the
       // copies of the tile after it (or, at the last tile, of the next item's first tile)
+      uint32_t e_cur = (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1]);   // the entry of the current tile
+      uint32_t e_nxt = 0;                                                        // of the next one, set by tile_head
+      uint16_t e_ahead = mlist[2];                                               // per lane, not yet made uniform
       // `may_be_last`: the item's last tile is an own-segment tile (merge_pair_lists_kernel ends every list with one),
       // so the loop over the permuted tiles always has a next entry to request and carries no code for the next item's
       // first tile
@@ -420,8 +423,12 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
         __syncthreads();                      // every share has; every wave is done with tile it - 1
         if (PBS_UNLIKELY(it == claim_it + 1)) adopt_next();
         if (PBS_UNLIKELY(it == claim_it) && wave == 0 && lane_id_here() == 0) claim = atomicAdd(PBS_ARGS()->queue + vic, 1);
+        // the list entries are read from LDS one tile ahead of their use (the read's latency would otherwise sit in
+        // front of the copy requests of every tile): `e_ahead` holds entry it + 1, requested at the tile before
+        e_nxt = (uint32_t)__builtin_amdgcn_readfirstlane((int)e_ahead);
+        e_ahead = mlist[3 + it];
         if (!decltype(may_be_last)::value || PBS_LIKELY(it + 1 < n_tiles))
-          stage_entry(hb, (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[2 + it]), bufx ^ 0x8000u, lane, lane_off);
+          stage_entry(hb, e_nxt, bufx ^ 0x8000u, lane, lane_off);
         else if (has_nxt && (careful_only || n_tiles >= 3))   // shorter items: after the loop, once the list has landed
           stage_entry(head_base(PBS_ARGS(), nxt / npair), (uint32_t)__builtin_amdgcn_readfirstlane((int)nlist[1]), bufx ^ 0x8000u, lane, lane_off);
       };
@@ -524,42 +531,38 @@ __global__ __launch_bounds__(512, 2) void sparse_attn_kernel(AttnArgs a) {
       // pass: a loop whose body updates the 64 accumulator registers on one path only keeps them in place, where
       // alternative tile bodies inside one loop cost a copy of all of them per tile (and the registers for it).
       int it = 0;
-      auto entry = [&](int i) __attribute__((always_inline)) { return (uint32_t)__builtin_amdgcn_readfirstlane((int)mlist[1 + i]); };
       if (PBS_UNLIKELY(careful_only)) {
-        for (; it < n_tiles; ++it, next_buffers()) {
-          const uint32_t ent = entry(it);
+        for (; it < n_tiles; ++it, next_buffers(), e_cur = e_nxt) {
           tile_head(it, any_tile);
-          if (!(ent & use_bit) || !qb_valid) continue;
-          careful_tile(ent, (ent & ENT_ORIG) && (int)(ent & ENT_KB) == qb);
+          if (!(e_cur & use_bit) || !qb_valid) continue;
+          careful_tile(e_cur, (e_cur & ENT_ORIG) && (int)(e_cur & ENT_KB) == qb);
         }
       } else {
-        for (; it < n_tiles; ++it, next_buffers()) {          // permuted tiles
-          const uint32_t ent = entry(it);
-          if (PBS_UNLIKELY(ent & ENT_ORIG)) break;
+        for (; it < n_tiles; ++it, next_buffers(), e_cur = e_nxt) {          // permuted tiles
+          if (PBS_UNLIKELY(e_cur & ENT_ORIG)) break;
           tile_head(it, not_the_last);
-          if (PBS_UNLIKELY(!(ent & use_bit) || !qb_valid)) continue;
+          if (PBS_UNLIKELY(!(e_cur & use_bit) || !qb_valid)) continue;
           if (PBS_UNLIKELY(first)) first_reference();
           fast_tile<false, PREFETCH_SLOTS, false>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
         }
-        for (; it < n_tiles; ++it, next_buffers()) {          // own-segment tiles before the diagonal: every key visible
-          const uint32_t ent = entry(it);
-          if ((int)(ent & ENT_KB) >= qb) break;
+        for (; it < n_tiles; ++it, next_buffers(), e_cur = e_nxt) {          // own-segment tiles before the diagonal: every key visible
+          if ((int)(e_cur & ENT_KB) >= qb) break;
           tile_head(it, any_tile);
-          if (!(ent & use_bit) || !qb_valid) continue;
+          if (!(e_cur & use_bit) || !qb_valid) continue;
           if (first) first_reference();
           fast_tile<false, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
         }
-        if (it < n_tiles && (int)(entry(it) & ENT_KB) == qb) {   // the diagonal tile
-          const uint32_t ent = entry(it);
+        if (it < n_tiles && (int)(e_cur & ENT_KB) == qb) {   // the diagonal tile
           tile_head(it, any_tile);
-          if ((ent & use_bit) && qb_valid) {
-            if (first || !all_seen) careful_tile(ent, true);
+          if ((e_cur & use_bit) && qb_valid) {
+            if (first || !all_seen) careful_tile(e_cur, true);
             else fast_tile<true, PREFETCH_SLOTS, true>(o, qf, ka, va, c_log2, m_ref, l_row, poisoned, wq);
           }
           ++it;
           next_buffers();
+          e_cur = e_nxt;
         }
-        for (; it < n_tiles; ++it, next_buffers()) tile_head(it, any_tile);   // tiles of the pair's other block only
+        for (; it < n_tiles; ++it, next_buffers(), e_cur = e_nxt) tile_head(it, any_tile);   // tiles of the pair's other block only
       }
       if (!careful_only && n_tiles < 3) {
         if (n_tiles < 2) {
