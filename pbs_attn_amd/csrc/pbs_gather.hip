@@ -50,33 +50,59 @@ __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float 
   const int32_t* idx = a.idx + (int64_t)bh * a.nb * BS + kb * BS;
   uint16_t* kdst = a.perm_k + ((int64_t)bh * a.nb + kb) * BS * D;
 
-  float acc[8];
+  // Every load of the block is requested before the first is used: a workgroup's rows are then in flight together
+  // (one pass at a time, a workgroup waits eight times for 4 or 8 KB).  Rows past the end of the sequence read
+  // row 0 and are zeroed afterwards, so that no load sits behind a branch.
+  int src[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = a.pool_max ? -INFINITY : 0.f;
-
+  for (int pass = 0; pass < 8; ++pass) src[pass] = idx[pass * 16 + rg];
+  u32x4 kv[8], vv[8];
 #pragma unroll
   for (int pass = 0; pass < 8; ++pass) {
-    const int i = pass * 16 + rg;
-    const int pos = kb * BS + i;
-    u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-    if (pos < a.S) {
-      const int src = idx[i];
-      kv = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)src * a.k_ss + c * 8);
-      if (!POOL_ONLY) vv = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)src * a.v_ss + c * 8);
-    }
-    if (!POOL_ONLY) __builtin_nontemporal_store(kv, reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
+    const bool live = kb * BS + pass * 16 + rg < a.S;
+    const int row = live ? src[pass] : 0;
+    kv[pass] = *reinterpret_cast<const u32x4*>(ksrc + (int64_t)row * a.k_ss + c * 8);
+    if (!POOL_ONLY) vv[pass] = *reinterpret_cast<const u32x4*>(vsrc + (int64_t)row * a.v_ss + c * 8);
+  }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float lo = bf16_bits_to_f32(kv[e] & 0xffffu), hi = bf16_bits_to_f32(kv[e] >> 16);
-      if (a.pool_max) {
-        acc[2 * e] = fmaxf(acc[2 * e], lo);
-        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], hi);
-      } else {
-        acc[2 * e] += lo;
-        acc[2 * e + 1] += hi;
+  for (int pass = 0; pass < 8; ++pass) {
+    const bool live = kb * BS + pass * 16 + rg < a.S;
+    if (!live) {
+      kv[pass] = (u32x4){0, 0, 0, 0};
+      if (!POOL_ONLY) vv[pass] = (u32x4){0, 0, 0, 0};
+    }
+  }
+
+  float acc[8];
+  if (a.pool_max) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = -INFINITY;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] = fmaxf(acc[2 * e], bf16_bits_to_f32(kv[pass][e] & 0xffffu));
+        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], bf16_bits_to_f32(kv[pass][e] >> 16));
       }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] += bf16_bits_to_f32(kv[pass][e] & 0xffffu);
+        acc[2 * e + 1] += bf16_bits_to_f32(kv[pass][e] >> 16);
+      }
+  }
+  if (!POOL_ONLY) {
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+      const int i = pass * 16 + rg;
+      __builtin_nontemporal_store(kv[pass], reinterpret_cast<u32x4*>(kdst + i * D + c * 8));
       // stage V row-major (4-byte stores: the padded pitch keeps them aligned)
-      if (!POOL_ONLY) *reinterpret_cast<uint32_t*>(&vt[i * VT_PITCH + c * 8 + 2 * e]) = vv[e];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) *reinterpret_cast<uint32_t*>(&vt[i * VT_PITCH + c * 8 + 2 * e]) = vv[pass][e];
     }
   }
 #pragma unroll
@@ -106,11 +132,50 @@ __device__ __forceinline__ void gather_block(GatherArgs& a, uint16_t* vt, float 
   }
 }
 
+// Launch order.  The query heads of a KV group read the same keys (and values) in different orders, and a permuted
+// block only holds rows of its own segment.  Workgroups are handed to the XCDs round-robin in launch order (x
+// fastest), so the grid is (8, members of a task group, groups / 8): the workgroups of one task group -- CHUNK
+// consecutive blocks of every query head of one KV head -- have the same blockIdx.x, run on one XCD at about the same
+// time, and the chunk's rows come from HBM once for the whole group (for segments up to the chunk: 256 KB of K per
+// group at 128 keys a block).  Decoding costs one division: most workgroups of a filtered gather leave at once, and
+// what they run before that is the launch's time.
+constexpr int CHUNK = 8;
+
+struct TaskGroups {
+  int n_chunks;    // chunks of CHUNK blocks per head
+  int n_groups;    // B * Hkv * n_chunks; group = blockIdx.z * 8 + blockIdx.x
+  int G;           // query heads per KV head
+  dim3 grid;
+};
+
+__host__ inline TaskGroups task_groups(int B, int Hq, int Hkv, int nb, int kinds) {
+  TaskGroups t;
+  t.n_chunks = (nb + CHUNK - 1) / CHUNK;
+  t.n_groups = B * Hkv * t.n_chunks;
+  t.G = Hq / Hkv;
+  t.grid = dim3(8, (unsigned)(kinds * t.G * CHUNK), (unsigned)((t.n_groups + 7) / 8));
+  return t;
+}
+
+// (kind, head, block) of this workgroup; false if it has none (the last groups of a launch, the tail of a head's blocks)
+__device__ __forceinline__ bool my_task(const TaskGroups& t, int nb, int& kind, int& bh, int& blk) {
+  const int m = blockIdx.y, per_kind = t.G * CHUNK;
+  kind = m >= per_kind;
+  const int mm = m - (kind ? per_kind : 0);
+  const int tg = blockIdx.z * 8 + blockIdx.x;
+  const int bkv = tg / t.n_chunks, chunk = tg - bkv * t.n_chunks;
+  blk = chunk * CHUNK + (mm & (CHUNK - 1));
+  bh = bkv * t.G + mm / CHUNK;   // (b * Hkv + kvh) * G + head in group == b * Hq + h
+  return tg < t.n_groups && blk < nb;
+}
+
 template <bool POOL_ONLY>
-__global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a) {
+__global__ __launch_bounds__(256) void gather_kv_kernel(GatherArgs a, TaskGroups t) {
   __shared__ uint16_t vt[POOL_ONLY ? 2 : BS * VT_PITCH];
   __shared__ float pool[16][D];
-  gather_block<POOL_ONLY>(a, vt, pool, blockIdx.x, blockIdx.y);
+  int kind, bh, blk;
+  if (!my_task(t, a.nb, kind, bh, blk)) return;
+  gather_block<POOL_ONLY>(a, vt, pool, blk, bh);
 }
 
 
@@ -120,25 +185,37 @@ __device__ __forceinline__ void pool_q_block(float (&pool)[16][D], const uint16_
   const int b = bh / Hq, h = bh % Hq;
   const int rg = threadIdx.x >> 4, c = threadIdx.x & 15;
   const uint16_t* src = q + b * q_sb + h * q_sh;
-  float acc[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) acc[e] = pool_max ? -INFINITY : 0.f;
+  // all eight loads in flight before the first is used; rows past the end read the last row and count as zeros
+  u32x4 x[8];
 #pragma unroll
   for (int pass = 0; pass < 8; ++pass) {
     const int pos = qb * BS + pass * 16 + rg;
-    u32x4 x = {0, 0, 0, 0};
-    if (pos < S) x = *reinterpret_cast<const u32x4*>(src + (int64_t)pos * q_ss + c * 8);
+    x[pass] = *reinterpret_cast<const u32x4*>(src + (int64_t)min(pos, S - 1) * q_ss + c * 8);
+  }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float lo = bf16_bits_to_f32(x[e] & 0xffffu), hi = bf16_bits_to_f32(x[e] >> 16);
-      if (pool_max) {
-        acc[2 * e] = fmaxf(acc[2 * e], lo);
-        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], hi);
-      } else {
-        acc[2 * e] += lo;
-        acc[2 * e + 1] += hi;
+  for (int pass = 0; pass < 8; ++pass)
+    if (qb * BS + pass * 16 + rg >= S) x[pass] = (u32x4){0, 0, 0, 0};
+  float acc[8];
+  if (pool_max) {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = -INFINITY;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] = fmaxf(acc[2 * e], bf16_bits_to_f32(x[pass][e] & 0xffffu));
+        acc[2 * e + 1] = fmaxf(acc[2 * e + 1], bf16_bits_to_f32(x[pass][e] >> 16));
       }
-    }
+  } else {
+#pragma unroll
+    for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        acc[2 * e] += bf16_bits_to_f32(x[pass][e] & 0xffffu);
+        acc[2 * e + 1] += bf16_bits_to_f32(x[pass][e] >> 16);
+      }
   }
 #pragma unroll
   for (int e = 0; e < 8; ++e) pool[rg][c * 8 + e] = acc[e];
@@ -157,9 +234,9 @@ __global__ __launch_bounds__(256) void pool_q_kernel(const uint16_t* q, uint16_t
   pool_q_block(pool, q, pooled, Hq, S, nb, q_sb, q_sh, q_ss, pool_max, blockIdx.x, blockIdx.y);
 }
 
-// Both poolings of the block estimate in one launch, the two kinds of workgroup alternating in launch order: the
-// pooling of permuted key blocks waits on scattered 256-byte rows, the pooling of query blocks streams Q from
-// HBM; side by side each fills what the other leaves idle.
+// Both poolings of the block estimate in one launch: the pooling of permuted key blocks waits on scattered 256-byte
+// rows, the pooling of query blocks streams Q from HBM; side by side each fills what the other leaves idle.  A task
+// group's key poolings come first, then the query poolings of the same heads and blocks.
 struct PoolQArgs {
   const uint16_t* q;
   uint16_t* pooled_q;
@@ -167,12 +244,13 @@ struct PoolQArgs {
   int pool_max;
 };
 
-__global__ __launch_bounds__(256) void pool_qk_kernel(GatherArgs a, PoolQArgs p) {
+__global__ __launch_bounds__(256) void pool_qk_kernel(GatherArgs a, PoolQArgs p, TaskGroups t) {
   __shared__ uint16_t vt[2];
   __shared__ float pool[16][D];
-  const int bh = blockIdx.y >> 1;
-  if (blockIdx.y & 1) pool_q_block(pool, p.q, p.pooled_q, a.Hq, a.S, a.nb, p.q_sb, p.q_sh, p.q_ss, p.pool_max, blockIdx.x, bh);
-  else gather_block<true>(a, vt, pool, blockIdx.x, bh);
+  int kind, bh, blk;
+  if (!my_task(t, a.nb, kind, bh, blk)) return;
+  if (kind) pool_q_block(pool, p.q, p.pooled_q, a.Hq, a.S, a.nb, p.q_sb, p.q_sh, p.q_ss, p.pool_max, blk, bh);
+  else gather_block<true>(a, vt, pool, blk, bh);
 }
 
 }  // namespace
@@ -187,7 +265,6 @@ extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_in
   PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && v_sb % 8 == 0 && v_sh % 8 == 0 && v_ss % 8 == 0,
               "pbs_gather_kv: strides must keep rows 16-byte aligned");
   PBS_REQUIRE(((uintptr_t)k % 16) == 0 && ((uintptr_t)v % 16) == 0, "pbs_gather_kv: pointers must be 16-byte aligned");
-  PBS_REQUIRE(B * Hq <= 65535, "pbs_gather_kv: too many heads");
   GatherArgs a;
   a.k = (const uint16_t*)k; a.v = (const uint16_t*)v; a.idx = key_indices;
   a.perm_k = (uint16_t*)perm_k; a.perm_vt = (uint16_t*)perm_vt; a.pooled_k = (uint16_t*)pooled_k;
@@ -195,7 +272,9 @@ extern "C" int pbs_gather_kv(const void* k, const void* v, const int32_t* key_in
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss; a.v_sb = v_sb; a.v_sh = v_sh; a.v_ss = v_ss;
   a.pool_max = key_pool_max;
-  hipLaunchKernelGGL(gather_kv_kernel<false>, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
+  const TaskGroups t = task_groups(B, Hq, Hkv, a.nb, 1);
+  PBS_REQUIRE(t.grid.y <= 65535 && t.grid.z <= 65535, "pbs_gather_kv: too many heads or blocks");
+  hipLaunchKernelGGL(gather_kv_kernel<false>, t.grid, dim3(256), 0, (hipStream_t)stream, a, t);
   return pbs_check_launch("pbs_gather_kv");
 }
 
@@ -207,13 +286,14 @@ extern "C" int pbs_pool_k_permuted(const void* k, const int32_t* key_indices, vo
   PBS_REQUIRE(B > 0 && Hq > 0 && Hkv > 0 && Hq % Hkv == 0 && S > 0, "pbs_pool_k_permuted: bad shape");
   PBS_REQUIRE(k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 && ((uintptr_t)k % 16) == 0,
               "pbs_pool_k_permuted: rows must be 16-byte aligned");
-  PBS_REQUIRE(B * Hq <= 65535, "pbs_pool_k_permuted: too many heads");
   GatherArgs a = {};
   a.k = (const uint16_t*)k; a.idx = key_indices; a.pooled_k = (uint16_t*)pooled_k; a.needed = block_needed;
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
   a.k_sb = k_sb; a.k_sh = k_sh; a.k_ss = k_ss;
   a.pool_max = key_pool_max;
-  hipLaunchKernelGGL(gather_kv_kernel<true>, dim3(a.nb, B * Hq), dim3(256), 0, (hipStream_t)stream, a);
+  const TaskGroups t = task_groups(B, Hq, Hkv, a.nb, 1);
+  PBS_REQUIRE(t.grid.y <= 65535 && t.grid.z <= 65535, "pbs_pool_k_permuted: too many heads or blocks");
+  hipLaunchKernelGGL(gather_kv_kernel<true>, t.grid, dim3(256), 0, (hipStream_t)stream, a, t);
   return pbs_check_launch("pbs_pool_k_permuted");
 }
 
@@ -227,7 +307,6 @@ extern "C" int pbs_pool_blocks(const void* q, const void* k, const int32_t* key_
   PBS_REQUIRE(q_sb % 8 == 0 && q_sh % 8 == 0 && q_ss % 8 == 0 && k_sb % 8 == 0 && k_sh % 8 == 0 && k_ss % 8 == 0 &&
                   ((uintptr_t)q % 16) == 0 && ((uintptr_t)k % 16) == 0,
               "pbs_pool_blocks: rows must be 16-byte aligned");
-  PBS_REQUIRE(2 * B * Hq <= 65535, "pbs_pool_blocks: too many heads");
   GatherArgs a = {};
   a.k = (const uint16_t*)k; a.idx = key_indices; a.pooled_k = (uint16_t*)pooled_k; a.needed = block_needed;
   a.B = B; a.Hq = Hq; a.Hkv = Hkv; a.S = S; a.nb = (S + BS - 1) / BS;
@@ -236,7 +315,9 @@ extern "C" int pbs_pool_blocks(const void* q, const void* k, const int32_t* key_
   PoolQArgs p;
   p.q = (const uint16_t*)q; p.pooled_q = (uint16_t*)pooled_q; p.q_sb = q_sb; p.q_sh = q_sh; p.q_ss = q_ss;
   p.pool_max = query_pool_max;
-  hipLaunchKernelGGL(pool_qk_kernel, dim3(a.nb, 2 * B * Hq), dim3(256), 0, (hipStream_t)stream, a, p);
+  const TaskGroups t = task_groups(B, Hq, Hkv, a.nb, 2);
+  PBS_REQUIRE(t.grid.y <= 65535 && t.grid.z <= 65535, "pbs_pool_blocks: too many heads or blocks");
+  hipLaunchKernelGGL(pool_qk_kernel, t.grid, dim3(256), 0, (hipStream_t)stream, a, p, t);
   return pbs_check_launch("pbs_pool_blocks");
 }
 
