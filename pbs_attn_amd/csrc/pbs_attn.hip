@@ -79,11 +79,12 @@ typedef const __attribute__((address_space(4))) struct AttnArgs* ArgsPtr;
 // use_second << 15: the union of the two visit lists (ascending), then the own segments in ORIGINAL key order
 // (blocks first-of-segment .. query block, shared where the two blocks share a segment).  Block 0 also clears
 // the work counters of the attention kernel that follows on the stream.
-__global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __restrict__ cols, const int32_t* __restrict__ cnt,
+constexpr int MERGE_THREADS = 256;
+__global__ __launch_bounds__(MERGE_THREADS) void merge_pair_lists_kernel(const int32_t* __restrict__ cols, const int32_t* __restrict__ cnt,
                                                                uint16_t* __restrict__ plist, int* __restrict__ queue, int nb,
                                                                int bps, int cap, const uint8_t* __restrict__ own_needed) {
   __shared__ uint8_t flags0[4096], flags1[4096];
-  __shared__ int wsum[8];
+  __shared__ int wsum[MERGE_THREADS / 64];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int npair = (nb + 1) >> 1;
   const int bh = blockIdx.x / npair, pair = blockIdx.x % npair;
@@ -93,28 +94,28 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
   const int32_t* l1 = l0 + (second ? nb : 0);
   const int n0 = cnt[(int64_t)bh * nb + 2 * pair];
   const int n1 = second ? cnt[(int64_t)bh * nb + 2 * pair + 1] : 0;
-  constexpr int MAX_PER = 4096 / 512;
+  constexpr int MAX_PER = 4096 / MERGE_THREADS;
   int c0[MAX_PER], c1[MAX_PER];
 #pragma unroll
   for (int u = 0; u < MAX_PER; ++u) {
-    const int i = tid + 512 * u;
+    const int i = tid + MERGE_THREADS * u;
     c0[u] = i < n0 ? l0[i] : 0;
     c1[u] = i < n1 ? l1[i] : 0;
   }
-  for (int i = tid; i < nb; i += 512) {
+  for (int i = tid; i < nb; i += MERGE_THREADS) {
     flags0[i] = 0;
     flags1[i] = 0;
   }
   __syncthreads();
 #pragma unroll
   for (int u = 0; u < MAX_PER; ++u) {
-    const int i = tid + 512 * u;
+    const int i = tid + MERGE_THREADS * u;
     if (i < n0) flags0[c0[u]] = 1;
     if (i < n1) flags1[c1[u]] = 2;
   }
   __syncthreads();
   // compaction: thread t owns `per` consecutive key blocks; wave-level prefix, then wave totals
-  const int per = (nb + 511) / 512;
+  const int per = (nb + MERGE_THREADS - 1) / MERGE_THREADS;
   const int k0 = tid * per, k1 = min(k0 + per, nb);
   int c = 0;
   for (int kb = k0; kb < k1; ++kb) c += (flags0[kb] | flags1[kb]) ? 1 : 0;
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
   __syncthreads();
   int w = incl - c, total = 0;
 #pragma unroll
-  for (int x = 0; x < 8; ++x) {
+  for (int x = 0; x < MERGE_THREADS / 64; ++x) {
     const int ws = wsum[x];
     if (x < wave) w += ws;
     total += ws;
@@ -156,10 +157,10 @@ __global__ __launch_bounds__(512) void merge_pair_lists_kernel(const int32_t* __
     }
     return;
   }
-  if (tid < n_own) {
-    const int kb = sf0 + tid;
+  for (int t = tid; t < n_own; t += MERGE_THREADS) {
+    const int kb = sf0 + t;
     const int f = (kb <= qb0 ? 1 : 0) | ((second && kb >= sf1) ? 2 : 0);
-    out[1 + total + tid] = (uint16_t)(kb | ENT_ORIG | (f << 14));
+    out[1 + total + t] = (uint16_t)(kb | ENT_ORIG | (f << 14));
   }
   if (tid == 0) out[0] = (uint16_t)(total + n_own);
 }
@@ -801,7 +802,7 @@ static int sparse_attn_launch(const void* q, const void* perm_k, const void* per
     pbs_set_error("pbs_sparse_attn_fwd: cannot reserve %u bytes of LDS: %s", LDS_TOTAL, hipGetErrorString(attr));
     return (int)attr;
   }
-  hipLaunchKernelGGL(merge_pair_lists_kernel, dim3((unsigned)(a.BH * npair)), dim3(512), 0, (hipStream_t)stream, csr_cols, csr_cnt,
+  hipLaunchKernelGGL(merge_pair_lists_kernel, dim3((unsigned)(a.BH * npair)), dim3(MERGE_THREADS), 0, (hipStream_t)stream, csr_cols, csr_cnt,
                      (uint16_t*)((char*)workspace + 256), a.queue, a.nb, a.bps, a.cap, own_block_needed);
   hipLaunchKernelGGL(sparse_attn_kernel, dim3((unsigned)n_wg), dim3(512), LDS_TOTAL, (hipStream_t)stream, a);
   return pbs_check_launch("pbs_sparse_attn_fwd");
