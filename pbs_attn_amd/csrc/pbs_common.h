@@ -58,16 +58,22 @@ __device__ __forceinline__ uint64_t desc_stable_key(float v, uint32_t index) {
 }
 __device__ __forceinline__ float desc_key_value(uint64_t key) { return f32_from_orderable(~(uint32_t)(key >> 32)); }
 
-// In-place ascending bitonic sort of n_pow2 uint64 keys held in LDS by one workgroup.
+// In-place ascending bitonic sort of n_pow2 uint64 keys held in LDS by one workgroup (whole waves, any number).
+// Thread t of a stage exchanges elements lo(t) and lo(t) + stride.  The 64 threads t = 64 c .. 64 c + 63 belong to
+// one wave in every stage, and for strides up to 64 their pairs are exactly elements 128 c .. 128 c + 127: those
+// stages need no workgroup barrier between them (a wave's LDS accesses complete in order), only the stages with
+// longer strides and the first short one after them do -- 9 barriers instead of 55 for 1024 keys.
 __device__ __forceinline__ void bitonic_sort_lds(uint64_t* keys, int n_pow2) {
+  __syncthreads();
   for (int size = 2; size <= n_pow2; size <<= 1) {
-    for (int stride = size >> 1; stride > 0; stride >>= 1) {
-      __syncthreads();
+    for (int stride = size >> 1, sh = __builtin_ctz(size) - 1; stride > 0; stride >>= 1, --sh) {
+      if (stride >= 64) __syncthreads();            // stride 64: the data may come from a longer stride's stage
+      else __builtin_amdgcn_wave_barrier();
       for (int t = threadIdx.x; t < (n_pow2 >> 1); t += blockDim.x) {
-        int lo = ((t / stride) * (stride << 1)) + (t % stride);
-        int hi = lo + stride;
-        bool up = ((lo & size) == 0);
-        uint64_t a = keys[lo], b = keys[hi];
+        const int lo = ((t >> sh) << (sh + 1)) | (t & (stride - 1));
+        const int hi = lo + stride;
+        const bool up = ((lo & size) == 0);
+        const uint64_t a = keys[lo], b = keys[hi];
         if ((a > b) == up) {
           keys[lo] = b;
           keys[hi] = a;
