@@ -211,17 +211,39 @@ __global__ __launch_bounds__(256, 2) void score_kernel(ScoreArgs a) {
   }
 }
 
-__global__ __launch_bounds__(NQ) void score_reduce_kernel(ScoreArgs a) {
-  const int bh = blockIdx.x, qrow = threadIdx.x;
-  const float* p = a.part + (int64_t)bh * a.nchunk * NQ * 2;
-  float m = -INFINITY, l = 0.f;
-  for (int c = 0; c < a.nchunk; ++c) {
-    const float mc = p[((int64_t)c * NQ + qrow) * 2], lc = p[((int64_t)c * NQ + qrow) * 2 + 1];
-    const float m_new = fmaxf(m, mc);
-    l = l * __builtin_amdgcn_exp2f(m - m_new) + lc * __builtin_amdgcn_exp2f(mc - m_new);
-    m = m_new;
+// Folds the chunk partials of one head into row max + log2(row sum).  A row's chunks are spread over REDUCE_LANES
+// threads and taken in two passes -- the maximum over all chunks, then the sum of the chunk sums scaled to it -- so
+// that no term waits for the one before it: folded one after the other with a running maximum, a row is a chain of
+// `nchunk` dependent loads and exponentials (19 us for 64 chunks, as long as the two scoring passes of a short
+// sequence together).  The order of the additions is fixed: per thread ascending chunks, then ascending threads.
+constexpr int REDUCE_LANES = 8;
+
+__global__ __launch_bounds__(NQ * REDUCE_LANES) void score_reduce_kernel(ScoreArgs a) {
+  __shared__ float part[REDUCE_LANES][NQ];
+  const int bh = blockIdx.x, qrow = threadIdx.x % NQ, cl = threadIdx.x / NQ;
+  const float* p = a.part + (int64_t)bh * a.nchunk * NQ * 2 + qrow * 2;
+  float m = -INFINITY;
+#pragma unroll 8
+  for (int c = cl; c < a.nchunk; c += REDUCE_LANES) m = fmaxf(m, p[(int64_t)c * NQ * 2]);
+  part[cl][qrow] = m;
+  __syncthreads();
+#pragma unroll
+  for (int x = 0; x < REDUCE_LANES; ++x) m = fmaxf(m, part[x][qrow]);
+  __syncthreads();
+  float l = 0.f;
+#pragma unroll 8
+  for (int c = cl; c < a.nchunk; c += REDUCE_LANES) {
+    const float2 ml = *reinterpret_cast<const float2*>(p + (int64_t)c * NQ * 2);
+    l += ml.y * __builtin_amdgcn_exp2f(ml.x - m);
   }
-  a.stats[(int64_t)bh * NQ + qrow] = m + __builtin_amdgcn_logf(l);   // log base 2
+  part[cl][qrow] = l;
+  __syncthreads();
+  if (cl == 0) {
+    l = 0.f;
+#pragma unroll
+    for (int x = 0; x < REDUCE_LANES; ++x) l += part[x][qrow];
+    a.stats[(int64_t)bh * NQ + qrow] = m + __builtin_amdgcn_logf(l);   // log base 2
+  }
 }
 
 int chunks_for(int Sc, int chunk_keys) { return (Sc + chunk_keys - 1) / chunk_keys; }
@@ -291,7 +313,7 @@ int score_keys_launch(const char* who, const void* q, const void* k, float* scor
   dim3 grid(a.nchunk, B * Hkv);
   const dim3 block(Hq / Hkv > 1 ? 256 : 64);
   hipLaunchKernelGGL(score_kernel<false>, grid, block, LDS_SCORE_TOTAL, st, a);
-  hipLaunchKernelGGL(score_reduce_kernel, dim3(B * Hq), dim3(NQ), 0, st, a);
+  hipLaunchKernelGGL(score_reduce_kernel, dim3(B * Hq), dim3(NQ * REDUCE_LANES), 0, st, a);
   hipLaunchKernelGGL(score_kernel<true>, grid, block, LDS_SCORE_TOTAL, st, a);
   return pbs_check_launch(who);
 }
