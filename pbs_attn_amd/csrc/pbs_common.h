@@ -41,6 +41,14 @@ __device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
 }
 __device__ __forceinline__ float round_bf16(float f) { return bf16_bits_to_f32(f32_to_bf16_bits(f)); }
 
+// two values rounded to bf16 (nearest even) by one hardware conversion, returned as floats
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+__device__ __forceinline__ f32x2 hw_round_bf16x2(f32x2 x) {
+  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
+  return (f32x2){__builtin_bit_cast(float, packed << 16), __builtin_bit_cast(float, packed & 0xffff0000u)};
+}
+
 // ---- order-preserving float key ---------------------------------------------
 // ascending unsigned order == ascending float order; -0 == +0; NaN greatest.
 __device__ __forceinline__ uint32_t f32_orderable(float f) {

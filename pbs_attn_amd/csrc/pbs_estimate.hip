@@ -8,6 +8,7 @@
 // waves split the key-block tiles, first to find each row's (max, sum), then to
 // recompute the logits and write P with 128-byte row segments per store.
 #include "pbs_common.h"
+#include "pbs_div.h"
 #include "../../include/pbs_hip.h"   // the definitions below are checked against the public declarations
 
 namespace {
@@ -17,8 +18,14 @@ constexpr int D = 128;
 __device__ __forceinline__ bf16x8 load_frag(const uint16_t* row_ptr, int t, int half) {
   return *reinterpret_cast<const bf16x8*>(row_ptr + 16 * t + 8 * half);
 }
-__device__ __forceinline__ float logit_round(float acc, float sqrt_d) {
-  return round_bf16(round_bf16(acc) / sqrt_d);
+// two accumulators -> the logits a bf16 matmul followed by a bf16 division by sqrt(D) yields: round to bf16, divide
+// (the exact quotient, see pbs_div.h), round to bf16
+struct Divisor {
+  float b, y;   // sqrt(D) and its correctly rounded reciprocal
+};
+__device__ __forceinline__ f32x2 logit_round2(float acc0, float acc1, Divisor d) {
+  const f32x2 r = hw_round_bf16x2((f32x2){acc0, acc1});
+  return hw_round_bf16x2((f32x2){pbs_div_by_const(r.x, d.b, d.y), pbs_div_by_const(r.y, d.b, d.y)});
 }
 
 // number of candidate key blocks of query block qb (its candidates are key blocks 0 .. count - 1): the blocks
@@ -33,12 +40,12 @@ __device__ __forceinline__ int candidate_count(int qb, int bps) {
 // reads no others); otherwise all nb columns, zeros outside the candidates and NaN rows where there are none.
 template <bool CAUSAL, bool CANDIDATES_ONLY>
 __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_t* pooled_q, const uint16_t* pooled_k,
-                                                                   float* P, int nb, int bps, float sqrt_d) {
+                                                                   float* P, int nb, int bps, Divisor sqrt_d) {
   __shared__ float s_m[4][32], s_l[4][32];
   __shared__ float s_max[32], s_inv[32];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int j = lane & 31, half = lane >> 5;
-  const int qt = blockIdx.x, bh = blockIdx.y;
+  const int qt = (int)gridDim.x - 1 - (int)blockIdx.x, bh = blockIdx.y;   // the tiles with the most candidates start first
   const uint16_t* pq = pooled_q + (int64_t)bh * nb * D;
   const uint16_t* pk = pooled_k + (int64_t)bh * nb * D;
   float* out = P + (int64_t)bh * nb * nb;
@@ -66,10 +73,12 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
     for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(load_frag(row, t, half), qf[t], acc, 0, 0, 0);
     float v[16], mx = -INFINITY;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
+    for (int r = 0; r < 16; r += 2) {
       const int kb = 32 * kt + 8 * (r >> 2) + 4 * half + (r & 3);
-      v[r] = kb < cand_col ? logit_round(acc[r], sqrt_d) : -INFINITY;
-      mx = fmaxf(mx, v[r]);
+      const f32x2 l2 = logit_round2(acc[r], acc[r + 1], sqrt_d);
+      v[r] = kb < cand_col ? l2.x : -INFINITY;
+      v[r + 1] = kb + 1 < cand_col ? l2.y : -INFINITY;
+      mx = fmaxf(mx, fmaxf(v[r], v[r + 1]));
     }
     if (mx > -INFINITY) {
       const float m_new = fmaxf(m_run, mx);
@@ -114,16 +123,20 @@ __global__ __launch_bounds__(256) void block_logits_softmax_kernel(const uint16_
       for (int t = 0; t < 8; ++t) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(qa[t], load_frag(row, t, half), acc, 0, 0, 0);
     }
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int ql = 8 * (r >> 2) + 4 * half + (r & 3);
-      const int qb = 32 * qt + ql;
-      if (qb < nb && kb < nb) {
-        const int cand = candidate_count<CAUSAL>(qb, bps);
-        float p;
-        if (cand == 0) p = __uint_as_float(0x7fc00000u);
-        else if (kb < cand) p = __expf(logit_round(acc[r], sqrt_d) - s_max[ql]) * s_inv[ql];
-        else p = 0.f;
-        if (!CANDIDATES_ONLY || kb < cand) out[(int64_t)qb * nb + kb] = p;
+    for (int r = 0; r < 16; r += 2) {
+      const f32x2 l2 = logit_round2(acc[r], acc[r + 1], sqrt_d);
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int ql = 8 * (r >> 2) + 4 * half + (r & 3) + u;
+        const int qb = 32 * qt + ql;
+        if (qb < nb && kb < nb) {
+          const int cand = candidate_count<CAUSAL>(qb, bps);
+          float p;
+          if (cand == 0) p = __uint_as_float(0x7fc00000u);
+          else if (kb < cand) p = __expf((u ? l2.y : l2.x) - s_max[ql]) * s_inv[ql];
+          else p = 0.f;
+          if (!CANDIDATES_ONLY || kb < cand) out[(int64_t)qb * nb + kb] = p;
+        }
       }
     }
   }
@@ -138,7 +151,9 @@ int launch_block_logits(const char* who, bool causal, bool candidates_only, cons
   PBS_REQUIRE(head_dim == D, "%s: head_dim must be 128, got %d", who, head_dim);
   PBS_REQUIRE(rows > 0 && rows <= 65535 && nb > 0 && blocks_per_segment > 0, "%s: bad shape", who);
   const dim3 grid((nb + 31) / 32, rows);
-  const float sqrt_d = (float)sqrt((double)head_dim);
+  Divisor sqrt_d;
+  sqrt_d.b = (float)sqrt((double)head_dim);
+  sqrt_d.y = (float)(1.0 / (double)sqrt_d.b);   // the correctly rounded reciprocal for head_dim 128 (tests/c_abi/div_check.c)
   if (candidates_only)
     hipLaunchKernelGGL((block_logits_softmax_kernel<false, true>), grid, dim3(256), 0, (hipStream_t)stream, (const uint16_t*)pooled_q,
                        (const uint16_t*)pooled_k, block_attn_scores, nb, blocks_per_segment, sqrt_d);

@@ -42,12 +42,6 @@ __device__ __forceinline__ bf16x8 load_frag(const uint16_t* row_ptr, int t, int 
 // bf16, scale (multiplication by the reciprocal; it differs from the true quotient by at most one fp32 ulp,
 // which survives the second bf16 rounding only for values within 2^-16 of a tie), round to bf16.
 // Hardware conversions (round to nearest even), two values per conversion instruction.
-typedef __attribute__((ext_vector_type(2))) float f32x2;
-typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-__device__ __forceinline__ f32x2 hw_round_bf16x2(f32x2 x) {
-  const uint32_t packed = __builtin_bit_cast(uint32_t, __builtin_convertvector(x, bf16x2));
-  return (f32x2){__builtin_bit_cast(float, packed << 16), __builtin_bit_cast(float, packed & 0xffff0000u)};
-}
 __device__ __forceinline__ f32x2 logit2(float acc0, float acc1, float inv_sqrt_d) {
   const f32x2 r = hw_round_bf16x2((f32x2){acc0, acc1});
   return hw_round_bf16x2((f32x2){r.x * inv_sqrt_d, r.y * inv_sqrt_d});

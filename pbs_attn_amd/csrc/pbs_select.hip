@@ -450,10 +450,13 @@ __device__ __forceinline__ void select_row_by_wave(const SelectArgs& a, int64_t 
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
   int base = 0;
-  for (int kb0 = 0; kb0 < nb; kb0 += 64) {
+  // without mask outputs only the blocks of earlier segments matter: they are what the visit list and the gather's
+  // filter hold
+  const int kb_end = (a.sel_mask || a.final_mask) ? nb : seg_first;
+  for (int kb0 = 0; kb0 < kb_end; kb0 += 64) {
     const int kb = kb0 + lane;
     bool visit = false;
-    if (kb < nb) {
+    if (kb < kb_end) {
       const bool own = kb >= seg_first && kb < seg_end;
       const uint8_t sf = flag[kb];
       if (a.sel_mask) a.sel_mask[row_off + kb] = sf;
